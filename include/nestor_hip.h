@@ -1,0 +1,262 @@
+/*
+ * nestor_hip.h -- C ABI of libnestor_hip.so, the gfx950 (MI355X) kernels behind
+ * Nestor's routed hybrid expert-MLP path.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless the name ends in _host.
+ *   - Every entry point returns 0 on success or a negative NESTOR_HIP_E* code;
+ *     nothing throws across the boundary and nothing allocates: outputs and
+ *     workspaces are caller-owned.
+ *   - `stream` is a hipStream_t passed as void*; work is enqueued, never
+ *     synchronised.  No entry point reads device memory back to the host.
+ *   - Index maps are int64 and segment ends (`offs`) int32, the widths the
+ *     reference plan uses (nestor/backbones/grouped_mm.py:197-219,272-277).
+ *   - Row-major tensors; a "bank" is one expert of a stacked weight tensor.
+ *
+ * Each declaration cites the reference interface it stands in for (paths are
+ * relative to the reference checkout).
+ */
+#ifndef NESTOR_HIP_H_
+#define NESTOR_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NESTOR_HIP_ABI_VERSION 1
+
+/* status codes */
+#define NESTOR_HIP_OK 0
+#define NESTOR_HIP_EINVAL (-22)   /* bad size / alignment / dtype code / null pointer */
+#define NESTOR_HIP_ENOSPC (-28)   /* workspace too small */
+#define NESTOR_HIP_ELAUNCH (-5)   /* the HIP runtime refused the launch */
+#define NESTOR_HIP_ERANGE (-34)   /* size beyond what the kernels support */
+
+/* element type codes */
+#define NESTOR_HIP_F32 0
+#define NESTOR_HIP_BF16 1
+
+/* Row alignment of every expert segment in the padded layout
+ * (GROUPED_MM_ALIGN, nestor/backbones/grouped_mm.py:61). */
+#define NESTOR_HIP_ROW_ALIGN 16
+
+/* Rows covered by one tile of the device-side tile table (see
+ * nestor_hip_index_build / nestor_hip_tile_schedule). */
+#define NESTOR_HIP_TILE_M 128
+
+int nestor_hip_abi_version(void);
+const char* nestor_hip_strerror(int code);
+
+/* ------------------------------------------------------------------------
+ * Dispatch index build  (nestor/backbones/grouped_mm.py:222-321, _dispatch_plan)
+ *
+ * From the flat token-major bank ids of the routed rows, builds in three
+ * launches what the reference builds with argsort + scatter_add + two cumsums
+ * + the map cascade: the stable sort permutation `order`, per-bank `counts`,
+ * `raw_starts` / `padded_starts` (exclusive cumsums of counts and of counts
+ * rounded up to 16), `offs` (int32 segment ends, last one == rows_pad) and the
+ * five maps row_dest / pad_token / pad_src_row / eid_pad / pad_valid with slack
+ * entries zero.  rows_pad must equal ceil16(rows) + 16 * num_banks.
+ *
+ * capacity <= 0: dropless (the reference's behaviour).  capacity > 0: a row
+ * whose stable rank inside its bank is >= capacity gets no padded slot; its
+ * row_dest is rows_pad - 1 (always a slack row) and row_kept (optional,
+ * uint8[rows]) is 0.  counts / raw_starts / order always describe ALL rows;
+ * padded_starts / offs describe the kept rows.
+ *
+ * tile_table (int32[3 * max_tiles + 1]) receives the tile table the grouped
+ * GEMMs walk, laid out bank[max_tiles] | row0[max_tiles] | nrows[max_tiles] |
+ * num_tiles: tile t covers rows [row0[t], row0[t] + nrows[t]) of bank[t], with
+ * nrows <= NESTOR_HIP_TILE_M and never crossing a segment end; bank == -1
+ * marks a tile that lies wholly in the slack tail behind the last segment
+ * (outputs are zero-filled, no product is formed).  max_tiles must be
+ * >= nestor_hip_max_tiles(rows_pad, num_banks).
+ * ---------------------------------------------------------------------- */
+size_t nestor_hip_index_build_workspace_bytes(int64_t rows, int32_t num_banks);
+int64_t nestor_hip_max_tiles(int64_t rows_pad, int32_t num_banks);
+int nestor_hip_index_build(
+    const int64_t* expert_ids, int64_t rows, int32_t num_banks, int32_t slots,
+    int64_t rows_pad, int64_t capacity, int32_t valid_dtype,
+    int64_t* order, int64_t* counts, int64_t* raw_starts, int64_t* padded_starts,
+    int32_t* offs,
+    int64_t* row_dest, int64_t* pad_token, int64_t* pad_src_row, int64_t* eid_pad,
+    void* pad_valid, uint8_t* row_kept /* nullable */,
+    int32_t* tile_table, int64_t max_tiles,
+    void* workspace, size_t workspace_bytes, void* stream);
+
+/* The reference's fused map kernel boundary, argument for argument
+ * (nestor/backbones/triton_dispatch.py:109-160, build_dispatch_maps): order,
+ * padded_starts and raw_starts come from the caller.  Slack entries of the
+ * four rows_pad-long maps are written as zero by this call (the reference
+ * zero-initialises them in its wrapper). */
+int nestor_hip_build_dispatch_maps(
+    const int64_t* expert_ids, const int64_t* order,
+    const int64_t* padded_starts, const int64_t* raw_starts,
+    int64_t rows, int32_t num_banks, int32_t slots, int64_t rows_pad,
+    int32_t valid_dtype,
+    int64_t* row_dest, int64_t* pad_token, int64_t* pad_src_row, int64_t* eid_pad,
+    void* pad_valid, void* stream);
+
+/* Tile table from segment ends alone, for callers that only hold `offs`
+ * (segment_mm's contract, nestor/backbones/grouped_mm.py:83-104).  Every row
+ * up to offs[num_banks-1] belongs to a bank, so no tile is marked -1. */
+int nestor_hip_tile_schedule(
+    const int32_t* offs, int32_t num_banks,
+    int32_t* tile_table, int64_t max_tiles, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Row moves
+ * ---------------------------------------------------------------------- */
+
+/* x_pad[p,:] = pad_valid[p] ? bf16(x[pad_token[p],:]) : 0
+ * (nestor/backbones/triton_expert.py:509-539 dispatch_rows; kernel
+ * nestor/backbones/triton_packed.py:113-139).  dim % 8 == 0. */
+int nestor_hip_dispatch_rows_fwd(
+    const void* x, int32_t x_dtype, const int64_t* pad_token,
+    const void* pad_valid, int32_t valid_dtype,
+    void* x_pad /* bf16 [rows_pad, dim] */, int64_t rows_pad, int64_t dim,
+    void* stream);
+
+/* grad_x[t,:] = sum_{j<slots} grad_pad[row_dest[t*slots+j],:], fp32 sum,
+ * written in x's dtype (nestor/backbones/triton_packed.py:142-169,444-463). */
+int nestor_hip_dispatch_rows_bwd(
+    const void* grad_pad /* bf16 [rows_pad, dim] */, const int64_t* row_dest,
+    void* grad_x, int32_t x_dtype, int64_t num_tokens, int32_t slots, int64_t dim,
+    void* stream);
+
+/* out = bf16( f32(bf16(silu_f32(gate))) * f32(up) ), two roundings
+ * (nestor/backbones/triton_expert.py:149-176).  up/gate rows have stride
+ * `stride_in` elements, out rows `stride_out`; the fused up|gate layout is
+ * gate = up + hidden, stride_in = 2*hidden (:391-402).  hidden % 8 == 0. */
+int nestor_hip_swiglu_fwd(
+    const void* up, const void* gate, void* out,
+    int64_t rows, int64_t hidden, int64_t stride_in, int64_t stride_out,
+    void* stream);
+
+/* grad_up = bf16(go*act), grad_gate = bf16(f32(bf16(go*up)) * s*(1+g*(1-s)))
+ * (nestor/backbones/triton_expert.py:179-217). */
+int nestor_hip_swiglu_bwd(
+    const void* grad_out, const void* up, const void* gate,
+    void* grad_up, void* grad_gate,
+    int64_t rows, int64_t hidden, int64_t stride_in, int64_t stride_out,
+    int64_t stride_g, void* stream);
+
+/* out[r, 0:h] = bf16(a[r,:]), out[r, h:2h] = bf16(b[r,:])
+ * (nestor/backbones/triton_expert.py:220-243,542-559 cat_cast). */
+int nestor_hip_cat_cast_fwd(
+    const float* a, const float* b, void* out /* bf16 [rows, 2h] */,
+    int64_t rows, int64_t hidden, void* stream);
+/* ga[r,:] = f32(g[r,0:h]), gb[r,:] = f32(g[r,h:2h])  (:245-268). */
+int nestor_hip_cat_cast_bwd(
+    const void* g /* bf16 [rows, 2h] */, float* ga, float* gb,
+    int64_t rows, int64_t hidden, void* stream);
+
+/* out[o,:] = sum_{e<group} term(f32(y_pad[row_dest[o*group+e],:]) * w[o*group+e]),
+ * fp32 accumulate; round_term != 0 rounds every term to out_dtype first
+ * (nestor/backbones/triton_expert.py:271-302,456-480 combine_rows). */
+int nestor_hip_combine_rows_fwd(
+    const void* y_pad /* bf16 [rows_pad, dim] */, const int64_t* row_dest,
+    const void* weights, int32_t w_dtype,
+    void* out, int32_t out_dtype, int64_t n_out, int32_t group, int64_t dim,
+    int32_t round_term, void* stream);
+
+/* grad_y[p,:] = bf16(go[src/group,:] * w[src]) on valid rows, exact 0 on slack;
+ * grad_w[src] = sum_d go*y in fp32 when grad_w != NULL
+ * (nestor/backbones/triton_expert.py:304-344,482-503). grad_w entries of rows
+ * that own no padded slot are left untouched. */
+int nestor_hip_combine_rows_bwd(
+    const void* grad_out, int32_t go_dtype, const void* y_pad,
+    const int64_t* pad_src_row, const void* pad_valid, int32_t valid_dtype,
+    const void* weights, int32_t w_dtype,
+    void* grad_y /* bf16 [rows_pad, dim] */, float* grad_w /* nullable, [rows] */,
+    int64_t rows_pad, int32_t group, int64_t dim, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Grouped GEMMs (bf16 operands, fp32 accumulate on MFMA, bf16 results).
+ * All stand in for torch._grouped_mm(a, b, offs=offs) and its autograd as
+ * called from segment_mm (nestor/backbones/grouped_mm.py:83-104,417-450).
+ * They walk the tile table of nestor_hip_index_build / _tile_schedule, which
+ * carries the segment bounds.  K % 8 == 0 and N % 8 == 0.
+ * ---------------------------------------------------------------------- */
+
+/* out[r,:] = a[r,:] @ b[bank(r)]   a [rows_pad,K], b [E,K,N], out [rows_pad,N]. */
+int nestor_hip_grouped_gemm_nn(
+    const void* a, const void* b, void* out,
+    int64_t rows_pad, int64_t K, int64_t N, int32_t num_banks,
+    const int32_t* tile_table, int64_t max_tiles, void* stream);
+
+/* Up and gate projections as one launch over the two stacked banks
+ * w_up / w_gate [E,K,H] (nestor/backbones/expert_bank_stack.py:72-77), with
+ * SwiGLU in the epilogue: writes up_gate [rows_pad, 2H] (up | gate, each
+ * rounded to bf16, what the reference's fused up|gate GEMM returns,
+ * grouped_mm.py:409-417) when up_gate != NULL, and
+ * hidden [rows_pad, H] = swiglu(up_gate) with the rounding points of
+ * nestor_hip_swiglu_fwd. */
+int nestor_hip_grouped_gemm_upgate_swiglu(
+    const void* a, const void* w_up, const void* w_gate,
+    void* up_gate /* nullable */, void* hidden,
+    int64_t rows_pad, int64_t K, int64_t H, int32_t num_banks,
+    const int32_t* tile_table, int64_t max_tiles, void* stream);
+
+/* out[r,:] = a[r,:] @ b[bank(r)]^T   a [rows_pad,K], b [E,N,K], out [rows_pad,N]:
+ * the input-gradient GEMM of torch._grouped_mm's autograd. */
+int nestor_hip_grouped_gemm_nt(
+    const void* a, const void* b, void* out,
+    int64_t rows_pad, int64_t K, int64_t N, int32_t num_banks,
+    const int32_t* tile_table, int64_t max_tiles, void* stream);
+
+/* grad_x_pad = g_up_gate[:, :H] @ w_up[bank]^T + g_up_gate[:, H:] @ w_gate[bank]^T
+ * g_up_gate [rows_pad, 2H], w_up / w_gate [E,K,H], out [rows_pad,K]. */
+int nestor_hip_grouped_gemm_nt_upgate(
+    const void* g_up_gate, const void* w_up, const void* w_gate, void* out,
+    int64_t rows_pad, int64_t K, int64_t H, int32_t num_banks,
+    const int32_t* tile_table, int64_t max_tiles, void* stream);
+
+/* out[e] = a[seg(e),:]^T @ g[seg(e),:]   a [rows_pad,M] (row stride lda),
+ * g [rows_pad,N] (row stride ldg), out [E,M,N] (row stride ldo, bank stride
+ * bank_stride elements): the weight-gradient GEMM, contraction over the rows
+ * of each segment; banks with no rows get exact zeros
+ * (nestor/backbones/grouped_mm.py:477-479).  seg_start / seg_count
+ * (int64[E], e.g. padded_starts / counts) bound the contraction; when NULL
+ * the segments are taken from offs. */
+int nestor_hip_grouped_gemm_tn(
+    const void* a, int64_t lda, const void* g, int64_t ldg,
+    void* out, int64_t ldo, int64_t bank_stride,
+    int64_t rows_pad, int64_t M, int64_t N, int32_t num_banks,
+    const int32_t* offs, const int64_t* seg_start, const int64_t* seg_count,
+    void* stream);
+
+/* fp8 (OCP e4m3fn) weight variant of nestor_hip_grouped_gemm_nn for the
+ * weight-streaming inference regime: b_q [E,K,N] e4m3, scale [E,N] fp32 per
+ * output channel, out[r,n] = bf16( scale[bank,n] * sum_k a[r,k]*b_q[bank,k,n] ). */
+int nestor_hip_grouped_gemm_fp8w_nn(
+    const void* a, const void* b_q, const float* scale, void* out,
+    int64_t rows_pad, int64_t K, int64_t N, int32_t num_banks,
+    const int32_t* tile_table, int64_t max_tiles, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Router epilogue (eval-mode Router.forward after the score GEMM,
+ * nestor/backbones/nestor.py:558-593; batched over G routers,
+ * nestor/backbones/batched_router.py:210-227).
+ * scores [n, C] -> softmax_probs [n, C] (fp32; the caller narrows it when the
+ * reference would), topk_indices [n, k] (int64, descending biased score, ties
+ * broken towards the lower index), gates [n, C] (scores dtype, zero off the
+ * top-k and on rows with mask[row] == 0).
+ * gate_mode 0 = renorm, 1 = switch.  choice_bias [n_bias_rows, C] fp32 is
+ * indexed by row % n_bias_rows (1 row: one router; G rows: batched routers
+ * with n = T*G).  C <= 64, k <= 8.
+ * ---------------------------------------------------------------------- */
+int nestor_hip_router_topk(
+    const void* scores, int32_t dtype, const float* choice_bias, int32_t n_bias_rows,
+    const uint8_t* mask /* nullable, [n] */,
+    float* softmax_probs, int64_t* topk_indices, void* gates,
+    int64_t n, int32_t num_choices, int32_t top_k, int32_t gate_mode,
+    void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NESTOR_HIP_H_ */

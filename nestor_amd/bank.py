@@ -1,0 +1,162 @@
+"""Expert modules and their stacked parameter ownership.
+
+``StackedExpertBank`` keeps the layout contract of
+nestor/backbones/expert_bank_stack.py:58-213 -- ``w_up`` / ``w_gate``
+``[E, d_in, hidden]`` (each expert's ``weight.t()``), ``w_down``
+``[E, hidden, d_out]``, optional bias banks -- so a state dict written by one
+side loads into the other.  ``SwigluExpert`` / ``Linear2`` are the minimal
+modules with the attribute surface the grouped path reads
+(``layers[0]``, ``layers[1]``, ``gate``, ``gated``, ``activation``;
+nestor/scaling/blocks.py:251-312).
+"""
+
+from __future__ import annotations
+
+import math
+from collections.abc import Sequence
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from nestor_amd.flags import stacked_banks_requested
+
+_ACTIVATIONS = {"silu": F.silu, "gelu": F.gelu, "relu": F.relu}
+
+
+class Linear2(nn.Module):
+    """A linear map with ``weight [out, in]`` and optional ``bias`` whose
+    parameters can later be re-pointed at views of a stacked owner."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = False) -> None:
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight = nn.Parameter(torch.empty(out_features, in_features))
+        self.bias = nn.Parameter(torch.zeros(out_features)) if bias else None
+        with torch.no_grad():
+            self.weight.normal_(0.0, 1.0 / math.sqrt(in_features))
+
+    def forward(self, x: Tensor) -> Tensor:
+        return F.linear(x, self.weight, self.bias)
+
+
+class SwigluExpert(nn.Module):
+    """``down(act(gate(x)) * up(x))``; up/down are ``layers[0]`` / ``layers[1]``."""
+
+    gated = True
+
+    def __init__(self, input_dim: int, hidden_dim: int, output_dim: int,
+                 activation: str = "silu", bias: bool = False) -> None:
+        super().__init__()
+        self.input_dim, self.output_dim = input_dim, output_dim
+        self.hidden_dims = [hidden_dim]
+        self.activation = activation
+        self.layers = nn.ModuleList(
+            [Linear2(input_dim, hidden_dim, bias), Linear2(hidden_dim, output_dim, bias)]
+        )
+        self.gate = Linear2(input_dim, hidden_dim, False)
+        self._activation_fn = _ACTIVATIONS[activation]
+
+    def forward(self, x: Tensor) -> Tensor:
+        return self.layers[1](self._activation_fn(self.gate(x)) * self.layers[0](x))
+
+
+class StackedExpertBank(nn.Module):
+    """One bank of shape-identical experts owned as stacked parameters."""
+
+    def __init__(self, experts: Sequence[nn.Module]) -> None:
+        super().__init__()
+        first = experts[0]
+        if len(first.layers) != 2:
+            raise ValueError("StackedExpertBank expects 2-layer (single-hidden) experts.")
+        gated = bool(getattr(first, "gated", False))
+        biased = first.layers[0].bias is not None
+        for e in experts:
+            if bool(getattr(e, "gated", False)) != gated or len(e.layers) != 2:
+                raise ValueError("StackedExpertBank expects a structurally uniform bank.")
+            if any((lin.bias is not None) != biased for lin in e.layers):
+                raise ValueError("StackedExpertBank expects uniform bias presence.")
+            if gated and e.gate.bias is not None:
+                raise ValueError("StackedExpertBank expects bias-free gates (standard SwiGLU).")
+        self.num_experts = len(experts)
+        self.gated = gated
+
+        def owner(tensors: list[Tensor]) -> nn.Parameter:
+            with torch.no_grad():
+                return nn.Parameter(torch.stack(tensors).contiguous())
+
+        self.w_up = owner([e.layers[0].weight.t() for e in experts])
+        self.w_gate = owner([e.gate.weight.t() for e in experts]) if gated else None
+        self.w_down = owner([e.layers[1].weight.t() for e in experts])
+        self.b_up = owner([e.layers[0].bias for e in experts]) if biased else None
+        self.b_down = owner([e.layers[1].bias for e in experts]) if biased else None
+        self.install_views(experts)
+
+    def install_views(self, experts: Sequence[nn.Module]) -> None:
+        """Re-point every expert's ``weight`` / ``bias`` at a view of the owners;
+        the per-expert entries leave ``_parameters`` so the model exposes each
+        bank once.  Re-run after any ``_apply`` (``.to()`` / ``.cuda()``)."""
+
+        for i, e in enumerate(experts):
+            pairs = [(e.layers[0], self.w_up), (e.layers[1], self.w_down)]
+            if self.gated:
+                pairs.append((e.gate, self.w_gate))
+            for linear, bank in pairs:
+                linear._parameters.pop("weight", None)
+                linear.weight = bank[i].t()
+            if self.b_up is not None:
+                for linear, bank in ((e.layers[0], self.b_up), (e.layers[1], self.b_down)):
+                    linear._parameters.pop("bias", None)
+                    linear.bias = bank[i]
+
+    def cast(self, dtype: torch.dtype) -> tuple[Tensor, Tensor | None, Tensor]:
+        """``(w_up, w_gate, w_down)`` in the GEMM dtype, one cast each (none when
+        the owners already are that dtype)."""
+
+        return (
+            self.w_up.to(dtype),
+            self.w_gate.to(dtype) if self.w_gate is not None else None,
+            self.w_down.to(dtype),
+        )
+
+
+class StackedBanksMixin:
+    """Declares banks at construction, stacks them on request, and re-installs
+    the expert views after device / dtype moves
+    (nestor/backbones/expert_bank_stack.py:216-282)."""
+
+    def _declare_expert_banks(self, banks) -> None:
+        self._stacked_bank_specs = []
+        self._stacked_view_sources = []
+        for name, experts in banks:
+            setattr(self, name, None)
+            if experts:
+                self._stacked_bank_specs.append((name, list(experts)))
+
+    def _consolidate_expert_banks(self) -> int:
+        done = 0
+        for name, experts in getattr(self, "_stacked_bank_specs", []):
+            if getattr(self, name, None) is None:
+                bank = StackedExpertBank(experts)
+                setattr(self, name, bank)
+                self._stacked_view_sources.append((bank, experts))
+                done += 1
+        return done
+
+    def _apply(self, fn, recurse=True):
+        module = super()._apply(fn, recurse)
+        for bank, experts in getattr(self, "_stacked_view_sources", []):
+            bank.install_views(experts)
+        return module
+
+
+def consolidate_stacked_expert_banks(model: nn.Module, *, force: bool = False) -> int:
+    """Stack the declared banks of every module in ``model``; returns how many.
+    A no-op unless ``NESTOR_STACKED_EXPERT_BANKS=1`` or ``force``."""
+
+    if not (force or stacked_banks_requested()):
+        return 0
+    return sum(
+        m._consolidate_expert_banks() for m in model.modules() if isinstance(m, StackedBanksMixin)
+    )

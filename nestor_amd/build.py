@@ -1,0 +1,77 @@
+"""Compile ``libnestor_hip.so`` (gfx950) from ``nestor_amd/csrc`` with hipcc.
+
+The library has no Python or torch dependency: it is a plain C-ABI shared object
+(``include/nestor_hip.h``) built in-tree next to this file, so it travels with
+the source tree to any machine that runs the tests or the benchmark.
+
+Run ``python -m nestor_amd.build`` to (re)build.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+REPO_ROOT = PKG_DIR.parent
+CSRC = PKG_DIR / "csrc"
+INCLUDE = REPO_ROOT / "include"
+LIB_PATH = PKG_DIR / "libnestor_hip.so"
+
+SOURCES = ["index_build.hip", "rows.hip", "grouped_gemm.hip", "router.hip"]
+
+# -packed-fp32-ops off: the compiler must not form packed fp32 VALU ops.
+HIP_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    found = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(found):
+        raise RuntimeError("hipcc not found; cannot build libnestor_hip.so")
+    return found
+
+
+def _compile(src: str, obj_dir: Path) -> Path:
+    obj = obj_dir / (Path(src).stem + ".o")
+    cmd = [_hipcc(), *HIP_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", "-c", str(CSRC / src), "-o", str(obj)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build_library(verbose: bool = True) -> Path:
+    """Compile every HIP source and link ``libnestor_hip.so``; returns its path."""
+
+    obj_dir = PKG_DIR / "build"
+    obj_dir.mkdir(exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+        objs = list(pool.map(lambda s: _compile(s, obj_dir), SOURCES))
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stderr}")
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_library()

@@ -1,0 +1,134 @@
+// Router epilogue: softmax, biased top-k, gates -- one launch for a whole
+// [rows, choices] score block (all G private routers of a layer at once when
+// rows = tokens * G).  A row is spread over the smallest power-of-two group of
+// lanes that holds its choices, so a 64-lane wavefront routes 64 / group rows
+// and every reduction is a handful of xor-shuffles.
+//
+// Follows Router.forward in eval mode (nestor/backbones/nestor.py:558-593) and
+// its batched form (nestor/backbones/batched_router.py:210-227).  torch.topk
+// leaves the order of equal scores unspecified; here equal biased scores are
+// taken lowest index first.
+#include "common.hpp"
+
+namespace nestor {
+namespace {
+
+constexpr int kRouterBlock = 256;
+
+template <typename F>
+__device__ __forceinline__ float group_reduce(float v, int group, F op) {
+  for (int off = group >> 1; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+template <bool kF32>
+__global__ __launch_bounds__(kRouterBlock) void router_topk_kernel(
+    const void* __restrict__ scores, const float* __restrict__ choice_bias,
+    int n_bias_rows, const uint8_t* __restrict__ mask, float* __restrict__ probs,
+    int64_t* __restrict__ topk, void* __restrict__ gates, int64_t n, int num_choices,
+    int top_k, int gate_mode, int group_shift) {
+  const int group = 1 << group_shift;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * kRouterBlock + threadIdx.x;
+  const int64_t row = gid >> group_shift;
+  const int sub = static_cast<int>(gid & (group - 1));
+  const bool live = row < n && sub < num_choices;
+  const float ninf = -__builtin_inff();
+  float s = ninf, biased = ninf;
+  if (live) {
+    s = load_scalar(scores, row * num_choices + sub, kF32 ? NESTOR_HIP_F32 : NESTOR_HIP_BF16);
+    // scores (+ fp32 buffer) promote to fp32: one exact-then-rounded fp32 add.
+    biased = s + choice_bias[(row % n_bias_rows) * num_choices + sub];
+  }
+  auto fmax_op = [](float a, float b) { return a > b ? a : b; };
+  auto fadd_op = [](float a, float b) { return a + b; };
+  const float m = group_reduce(s, group, fmax_op);
+  const float e = live ? expf(s - m) : 0.0f;
+  const float denom = group_reduce(e, group, fadd_op);
+  const float prob = e / denom;
+  if (live) probs[row * num_choices + sub] = prob;
+
+  bool taken = false;
+  for (int j = 0; j < top_k; ++j) {
+    float best = taken ? ninf : biased;
+    int best_idx = (live && !taken) ? sub : 0x7fffffff;
+    for (int off = group >> 1; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(best, off, kWave);
+      const int oi = __shfl_xor(best_idx, off, kWave);
+      if (ov > best || (ov == best && oi < best_idx)) {
+        best = ov;
+        best_idx = oi;
+      }
+    }
+    if (live && sub == best_idx) {
+      taken = true;
+      topk[row * top_k + j] = sub;
+    }
+  }
+
+  float gate;
+  if (gate_mode == 1) {  // switch: full-softmax probability of the selected choices
+    gate = taken ? prob : 0.0f;
+  } else {               // renorm: softmax over the selected raw scores
+    const float m2 = group_reduce(taken ? s : ninf, group, fmax_op);
+    const float e2 = taken ? expf(s - m2) : 0.0f;
+    const float d2 = group_reduce(e2, group, fadd_op);
+    gate = taken ? e2 / d2 : 0.0f;
+  }
+  if (live) {
+    const bool valid = mask == nullptr || mask[row] != 0;
+    if constexpr (kF32) {
+      reinterpret_cast<float*>(gates)[row * num_choices + sub] = valid ? gate : 0.0f;
+    } else {
+      // gate is rounded to the score dtype before the validity product.
+      reinterpret_cast<uint16_t*>(gates)[row * num_choices + sub] =
+          valid ? static_cast<uint16_t>(f32_to_bf16_bits(gate)) : 0;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace nestor
+
+using namespace nestor;
+
+extern "C" int nestor_hip_router_topk(const void* scores, int32_t dtype,
+                                      const float* choice_bias, int32_t n_bias_rows,
+                                      const uint8_t* mask, float* softmax_probs,
+                                      int64_t* topk_indices, void* gates, int64_t n,
+                                      int32_t num_choices, int32_t top_k, int32_t gate_mode,
+                                      void* stream) {
+  if ((dtype != NESTOR_HIP_F32 && dtype != NESTOR_HIP_BF16) || num_choices <= 0 ||
+      num_choices > 64 || top_k <= 0 || top_k > num_choices || n_bias_rows <= 0 || n < 0 ||
+      (gate_mode != 0 && gate_mode != 1))
+    return NESTOR_HIP_EINVAL;
+  if (n == 0) return NESTOR_HIP_OK;
+  if (!scores || !choice_bias || !softmax_probs || !topk_indices || !gates)
+    return NESTOR_HIP_EINVAL;
+  int shift = 0;
+  while ((1 << shift) < num_choices) ++shift;
+  const int64_t threads = n << shift;
+  const unsigned blocks = static_cast<unsigned>(ceil_div(threads, kRouterBlock));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(router_topk_kernel<true>, dim3(blocks), dim3(kRouterBlock), 0, s,
+                       scores, choice_bias, n_bias_rows, mask, softmax_probs, topk_indices,
+                       gates, n, num_choices, top_k, gate_mode, shift);
+  else
+    hipLaunchKernelGGL(router_topk_kernel<false>, dim3(blocks), dim3(kRouterBlock), 0, s,
+                       scores, choice_bias, n_bias_rows, mask, softmax_probs, topk_indices,
+                       gates, n, num_choices, top_k, gate_mode, shift);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_abi_version(void) { return NESTOR_HIP_ABI_VERSION; }
+
+extern "C" const char* nestor_hip_strerror(int code) {
+  switch (code) {
+    case NESTOR_HIP_OK: return "ok";
+    case NESTOR_HIP_EINVAL: return "invalid argument (size, alignment, dtype code or null pointer)";
+    case NESTOR_HIP_ENOSPC: return "workspace too small";
+    case NESTOR_HIP_ELAUNCH: return "HIP kernel launch failed";
+    case NESTOR_HIP_ERANGE: return "size beyond what the kernels support";
+    default: return "unknown nestor_hip status";
+  }
+}

@@ -1,0 +1,382 @@
+// HBM-bound row kernels around the grouped GEMMs: dispatch gather (+ its
+// gather-sum backward), SwiGLU, the stacked-bank cat+cast, and the weighted
+// slot combine (+ backward).  One wavefront owns one row and moves it in
+// 16-byte pieces per lane, so every global access is a full 128-bit
+// transaction and a row's 64 lanes cover 1 KiB of contiguous memory at a time.
+// No float atomics anywhere: every output element has exactly one writer and a
+// fixed summation order.
+#include "common.hpp"
+
+namespace nestor {
+namespace {
+
+constexpr int kRowBlock = 256;
+constexpr int kRowsPerBlock = kRowBlock / kWave;
+
+__device__ __forceinline__ int64_t wave_row() {
+  return static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
+}
+
+// x_pad[p,:] = valid[p] ? bf16(x[pad_token[p],:]) : 0
+template <bool kXF32>
+__global__ __launch_bounds__(kRowBlock) void dispatch_fwd_kernel(
+    const void* __restrict__ x, const int64_t* __restrict__ pad_token,
+    const void* __restrict__ pad_valid, int valid_dtype, uint16_t* __restrict__ out,
+    int64_t rows_pad, int64_t dim) {
+  const int64_t p = wave_row();
+  if (p >= rows_pad) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  uint16_t* dst = out + p * dim;
+  if (!load_valid(pad_valid, p, valid_dtype)) {
+    const u32x4 zero = {0, 0, 0, 0};
+    for (int c = lane; c < chunks; c += kWave) st16(dst + c * 8, zero);
+    return;
+  }
+  const int64_t tok = pad_token[p];
+  for (int c = lane; c < chunks; c += kWave) {
+    if constexpr (kXF32) {
+      float f[8];
+      load8_as_f32<true>(x, tok * dim + c * 8, f);
+      st16(dst + c * 8, pack8(f));
+    } else {
+      st16(dst + c * 8, ld16(reinterpret_cast<const uint16_t*>(x) + tok * dim + c * 8));
+    }
+  }
+}
+
+// gx[t,:] = sum_j g[row_dest[t*slots+j],:]  (fp32 sum, slot order)
+template <bool kXF32>
+__global__ __launch_bounds__(kRowBlock) void dispatch_bwd_kernel(
+    const uint16_t* __restrict__ g, const int64_t* __restrict__ row_dest,
+    void* __restrict__ gx, int64_t num_tokens, int slots, int64_t dim) {
+  const int64_t t = wave_row();
+  if (t >= num_tokens) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  for (int c = lane; c < chunks; c += kWave) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int j = 0; j < slots; ++j) {
+      const int64_t r = row_dest[t * slots + j];
+      float f[8];
+      unpack8(ld16(g + r * dim + c * 8), f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += f[i];
+    }
+    store8_from_f32<kXF32>(gx, t * dim + c * 8, acc);
+  }
+}
+
+__device__ __forceinline__ float silu_rounded(float g) {
+  // ATen silu: x / (1 + exp(-x)) in fp32, rounded to the bf16 input dtype.
+  return round_bf16(g / (1.0f + __expf(-g)));
+}
+
+__global__ __launch_bounds__(kRowBlock) void swiglu_fwd_kernel(
+    const uint16_t* __restrict__ up, const uint16_t* __restrict__ gate,
+    uint16_t* __restrict__ out, int64_t rows, int64_t hidden, int64_t stride_in,
+    int64_t stride_out) {
+  const int64_t r = wave_row();
+  if (r >= rows) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(hidden / 8);
+  for (int c = lane; c < chunks; c += kWave) {
+    float u[8], g[8], o[8];
+    unpack8(ld16(up + r * stride_in + c * 8), u);
+    unpack8(ld16(gate + r * stride_in + c * 8), g);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = silu_rounded(g[i]) * u[i];
+    st16(out + r * stride_out + c * 8, pack8(o));
+  }
+}
+
+__global__ __launch_bounds__(kRowBlock) void swiglu_bwd_kernel(
+    const uint16_t* __restrict__ gout, const uint16_t* __restrict__ up,
+    const uint16_t* __restrict__ gate, uint16_t* __restrict__ gup,
+    uint16_t* __restrict__ ggate, int64_t rows, int64_t hidden, int64_t stride_in,
+    int64_t stride_out, int64_t stride_g) {
+  const int64_t r = wave_row();
+  if (r >= rows) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(hidden / 8);
+  for (int c = lane; c < chunks; c += kWave) {
+    float go[8], u[8], g[8], du[8], dg[8];
+    unpack8(ld16(gout + r * stride_g + c * 8), go);
+    unpack8(ld16(up + r * stride_in + c * 8), u);
+    unpack8(ld16(gate + r * stride_in + c * 8), g);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float e = __expf(-g[i]);
+      const float s = 1.0f / (1.0f + e);
+      const float act = round_bf16(g[i] / (1.0f + e));
+      du[i] = go[i] * act;
+      const float gact = round_bf16(go[i] * u[i]);
+      // ATen silu_backward: dy * s * (1 + x * (1 - s)) in fp32.
+      dg[i] = gact * s * (1.0f + g[i] * (1.0f - s));
+    }
+    st16(gup + r * stride_out + c * 8, pack8(du));
+    st16(ggate + r * stride_out + c * 8, pack8(dg));
+  }
+}
+
+__global__ __launch_bounds__(kRowBlock) void cat_cast_fwd_kernel(
+    const float* __restrict__ a, const float* __restrict__ b, uint16_t* __restrict__ out,
+    int64_t rows, int64_t hidden) {
+  const int64_t r = wave_row();
+  if (r >= rows) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(hidden / 8);
+  for (int c = lane; c < chunks; c += kWave) {
+    float f[8];
+    load8_as_f32<true>(a, r * hidden + c * 8, f);
+    st16(out + r * 2 * hidden + c * 8, pack8(f));
+    load8_as_f32<true>(b, r * hidden + c * 8, f);
+    st16(out + r * 2 * hidden + hidden + c * 8, pack8(f));
+  }
+}
+
+__global__ __launch_bounds__(kRowBlock) void cat_cast_bwd_kernel(
+    const uint16_t* __restrict__ g, float* __restrict__ ga, float* __restrict__ gb,
+    int64_t rows, int64_t hidden) {
+  const int64_t r = wave_row();
+  if (r >= rows) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(hidden / 8);
+  for (int c = lane; c < chunks; c += kWave) {
+    float f[8];
+    unpack8(ld16(g + r * 2 * hidden + c * 8), f);
+    store8_from_f32<true>(ga, r * hidden + c * 8, f);
+    unpack8(ld16(g + r * 2 * hidden + hidden + c * 8), f);
+    store8_from_f32<true>(gb, r * hidden + c * 8, f);
+  }
+}
+
+constexpr int kMaxGroup = 32;
+
+// out[o,:] = sum_e term(y[row_dest[o*group+e],:] * w[o*group+e])
+template <bool kOutF32>
+__global__ __launch_bounds__(kRowBlock) void combine_fwd_kernel(
+    const uint16_t* __restrict__ y, const int64_t* __restrict__ row_dest,
+    const void* __restrict__ weights, int w_dtype, void* __restrict__ out,
+    int64_t n_out, int group, int64_t dim, int round_term) {
+  const int64_t o = wave_row();
+  if (o >= n_out) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const bool round = round_term != 0 && !kOutF32;  // rounding to fp32 is the identity
+  for (int c = lane; c < chunks; c += kWave) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int e = 0; e < group; ++e) {
+      const int64_t r = o * group + e;
+      const int64_t p = row_dest[r];
+      const float w = load_scalar(weights, r, w_dtype);
+      float f[8];
+      unpack8(ld16(y + p * dim + c * 8), f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float term = f[i] * w;
+        if (round) term = round_bf16(term);
+        acc[i] += term;
+      }
+    }
+    store8_from_f32<kOutF32>(out, o * dim + c * 8, acc);
+  }
+}
+
+// gy[p,:] = bf16(go[src/group,:] * w[src]) * valid[p];  gw[src] = sum_d go*y
+template <bool kGoF32>
+__global__ __launch_bounds__(kRowBlock) void combine_bwd_kernel(
+    const void* __restrict__ gout, const uint16_t* __restrict__ y,
+    const int64_t* __restrict__ pad_src_row, const void* __restrict__ pad_valid,
+    int valid_dtype, const void* __restrict__ weights, int w_dtype,
+    uint16_t* __restrict__ gy, float* __restrict__ gw, int64_t rows_pad, int group,
+    int64_t dim) {
+  const int64_t p = wave_row();
+  if (p >= rows_pad) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  uint16_t* dst = gy + p * dim;
+  if (!load_valid(pad_valid, p, valid_dtype)) {
+    const u32x4 zero = {0, 0, 0, 0};
+    for (int c = lane; c < chunks; c += kWave) st16(dst + c * 8, zero);
+    return;
+  }
+  const int64_t src = pad_src_row[p];
+  const float w = load_scalar(weights, src, w_dtype);
+  const int64_t orow = src / group;
+  float dot = 0.0f;
+  for (int c = lane; c < chunks; c += kWave) {
+    float go[8], o[8];
+    load8_as_f32<kGoF32>(gout, orow * dim + c * 8, go);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = go[i] * w;
+    st16(dst + c * 8, pack8(o));
+    if (gw != nullptr) {
+      float f[8];
+      unpack8(ld16(y + p * dim + c * 8), f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dot += go[i] * f[i];
+    }
+  }
+  if (gw != nullptr) {
+    dot = wave_sum(dot);
+    if (lane == 0) gw[src] = dot;
+  }
+}
+
+inline unsigned row_blocks(int64_t rows) {
+  return static_cast<unsigned>(ceil_div(rows, kRowsPerBlock));
+}
+inline bool dtype_ok(int d) { return d == NESTOR_HIP_F32 || d == NESTOR_HIP_BF16; }
+
+}  // namespace
+}  // namespace nestor
+
+using namespace nestor;
+
+extern "C" int nestor_hip_dispatch_rows_fwd(const void* x, int32_t x_dtype,
+                                            const int64_t* pad_token,
+                                            const void* pad_valid, int32_t valid_dtype,
+                                            void* x_pad, int64_t rows_pad, int64_t dim,
+                                            void* stream) {
+  if (!dtype_ok(x_dtype) || !dtype_ok(valid_dtype) || dim <= 0 || dim % 8 != 0 ||
+      rows_pad < 0)
+    return NESTOR_HIP_EINVAL;
+  if (rows_pad == 0) return NESTOR_HIP_OK;
+  if (!x || !pad_token || !pad_valid || !x_pad) return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto* out = static_cast<uint16_t*>(x_pad);
+  if (x_dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(dispatch_fwd_kernel<true>, dim3(row_blocks(rows_pad)),
+                       dim3(kRowBlock), 0, s, x, pad_token, pad_valid, valid_dtype, out,
+                       rows_pad, dim);
+  else
+    hipLaunchKernelGGL(dispatch_fwd_kernel<false>, dim3(row_blocks(rows_pad)),
+                       dim3(kRowBlock), 0, s, x, pad_token, pad_valid, valid_dtype, out,
+                       rows_pad, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_dispatch_rows_bwd(const void* grad_pad, const int64_t* row_dest,
+                                            void* grad_x, int32_t x_dtype,
+                                            int64_t num_tokens, int32_t slots,
+                                            int64_t dim, void* stream) {
+  if (!dtype_ok(x_dtype) || dim <= 0 || dim % 8 != 0 || num_tokens < 0 || slots <= 0)
+    return NESTOR_HIP_EINVAL;
+  if (num_tokens == 0) return NESTOR_HIP_OK;
+  if (!grad_pad || !row_dest || !grad_x) return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto* g = static_cast<const uint16_t*>(grad_pad);
+  if (x_dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(dispatch_bwd_kernel<true>, dim3(row_blocks(num_tokens)),
+                       dim3(kRowBlock), 0, s, g, row_dest, grad_x, num_tokens, slots, dim);
+  else
+    hipLaunchKernelGGL(dispatch_bwd_kernel<false>, dim3(row_blocks(num_tokens)),
+                       dim3(kRowBlock), 0, s, g, row_dest, grad_x, num_tokens, slots, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_swiglu_fwd(const void* up, const void* gate, void* out,
+                                     int64_t rows, int64_t hidden, int64_t stride_in,
+                                     int64_t stride_out, void* stream) {
+  if (hidden <= 0 || hidden % 8 != 0 || stride_in % 8 != 0 || stride_out % 8 != 0 ||
+      stride_in < hidden || stride_out < hidden || rows < 0)
+    return NESTOR_HIP_EINVAL;
+  if (rows == 0) return NESTOR_HIP_OK;
+  if (!up || !gate || !out) return NESTOR_HIP_EINVAL;
+  hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(row_blocks(rows)), dim3(kRowBlock), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(up),
+                     static_cast<const uint16_t*>(gate), static_cast<uint16_t*>(out), rows,
+                     hidden, stride_in, stride_out);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_swiglu_bwd(const void* grad_out, const void* up,
+                                     const void* gate, void* grad_up, void* grad_gate,
+                                     int64_t rows, int64_t hidden, int64_t stride_in,
+                                     int64_t stride_out, int64_t stride_g, void* stream) {
+  if (hidden <= 0 || hidden % 8 != 0 || stride_in % 8 != 0 || stride_out % 8 != 0 ||
+      stride_g % 8 != 0 || stride_in < hidden || stride_out < hidden ||
+      stride_g < hidden || rows < 0)
+    return NESTOR_HIP_EINVAL;
+  if (rows == 0) return NESTOR_HIP_OK;
+  if (!grad_out || !up || !gate || !grad_up || !grad_gate) return NESTOR_HIP_EINVAL;
+  hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(row_blocks(rows)), dim3(kRowBlock), 0,
+                     static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(grad_out),
+                     static_cast<const uint16_t*>(up), static_cast<const uint16_t*>(gate),
+                     static_cast<uint16_t*>(grad_up), static_cast<uint16_t*>(grad_gate),
+                     rows, hidden, stride_in, stride_out, stride_g);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_cat_cast_fwd(const float* a, const float* b, void* out,
+                                       int64_t rows, int64_t hidden, void* stream) {
+  if (hidden <= 0 || hidden % 8 != 0 || rows < 0) return NESTOR_HIP_EINVAL;
+  if (rows == 0) return NESTOR_HIP_OK;
+  if (!a || !b || !out) return NESTOR_HIP_EINVAL;
+  hipLaunchKernelGGL(cat_cast_fwd_kernel, dim3(row_blocks(rows)), dim3(kRowBlock), 0,
+                     static_cast<hipStream_t>(stream), a, b, static_cast<uint16_t*>(out),
+                     rows, hidden);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_cat_cast_bwd(const void* g, float* ga, float* gb, int64_t rows,
+                                       int64_t hidden, void* stream) {
+  if (hidden <= 0 || hidden % 8 != 0 || rows < 0) return NESTOR_HIP_EINVAL;
+  if (rows == 0) return NESTOR_HIP_OK;
+  if (!g || !ga || !gb) return NESTOR_HIP_EINVAL;
+  hipLaunchKernelGGL(cat_cast_bwd_kernel, dim3(row_blocks(rows)), dim3(kRowBlock), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(g), ga,
+                     gb, rows, hidden);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_combine_rows_fwd(const void* y_pad, const int64_t* row_dest,
+                                           const void* weights, int32_t w_dtype, void* out,
+                                           int32_t out_dtype, int64_t n_out, int32_t group,
+                                           int64_t dim, int32_t round_term, void* stream) {
+  if (!dtype_ok(w_dtype) || !dtype_ok(out_dtype) || dim <= 0 || dim % 8 != 0 ||
+      group <= 0 || group > kMaxGroup || n_out < 0)
+    return NESTOR_HIP_EINVAL;
+  if (n_out == 0) return NESTOR_HIP_OK;
+  if (!y_pad || !row_dest || !weights || !out) return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto* y = static_cast<const uint16_t*>(y_pad);
+  if (out_dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(combine_fwd_kernel<true>, dim3(row_blocks(n_out)), dim3(kRowBlock),
+                       0, s, y, row_dest, weights, w_dtype, out, n_out, group, dim,
+                       round_term);
+  else
+    hipLaunchKernelGGL(combine_fwd_kernel<false>, dim3(row_blocks(n_out)), dim3(kRowBlock),
+                       0, s, y, row_dest, weights, w_dtype, out, n_out, group, dim,
+                       round_term);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_combine_rows_bwd(const void* grad_out, int32_t go_dtype,
+                                           const void* y_pad, const int64_t* pad_src_row,
+                                           const void* pad_valid, int32_t valid_dtype,
+                                           const void* weights, int32_t w_dtype,
+                                           void* grad_y, float* grad_w, int64_t rows_pad,
+                                           int32_t group, int64_t dim, void* stream) {
+  if (!dtype_ok(go_dtype) || !dtype_ok(valid_dtype) || !dtype_ok(w_dtype) || dim <= 0 ||
+      dim % 8 != 0 || group <= 0 || rows_pad < 0)
+    return NESTOR_HIP_EINVAL;
+  if (rows_pad == 0) return NESTOR_HIP_OK;
+  if (!grad_out || !pad_src_row || !pad_valid || !weights || !grad_y ||
+      (grad_w != nullptr && !y_pad))
+    return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto* y = static_cast<const uint16_t*>(y_pad);
+  auto* gy = static_cast<uint16_t*>(grad_y);
+  if (go_dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(combine_bwd_kernel<true>, dim3(row_blocks(rows_pad)),
+                       dim3(kRowBlock), 0, s, grad_out, y, pad_src_row, pad_valid,
+                       valid_dtype, weights, w_dtype, gy, grad_w, rows_pad, group, dim);
+  else
+    hipLaunchKernelGGL(combine_bwd_kernel<false>, dim3(row_blocks(rows_pad)),
+                       dim3(kRowBlock), 0, s, grad_out, y, pad_src_row, pad_valid,
+                       valid_dtype, weights, w_dtype, gy, grad_w, rows_pad, group, dim);
+  return launch_status();
+}

@@ -1,0 +1,237 @@
+"""Grouped expert dispatch on the HIP kernels: plan -> dispatch -> grouped GEMMs
+with SwiGLU -> weighted combine.
+
+Host-side mirror of nestor/backbones/grouped_mm.py: ``segment_mm`` (:83),
+``grouped_expert_rows`` (:453) and ``grouped_expert_combine`` (:558) keep their
+names, arguments and results.  What differs is underneath: the plan is one HIP
+index build instead of argsort + scatter cascade, every GEMM is an MFMA kernel
+driven by the plan's device-side tile table, and for bias-free SwiGLU banks
+under ``triton_fused`` the up and gate projections read the two stacked banks
+in place (no concatenated copy of the weights) with SwiGLU in the GEMM epilogue.
+
+The kernels compute in bfloat16 with fp32 accumulation; any other GEMM dtype is
+rejected, and CPU tensors are rejected by the ops themselves.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Sequence
+from typing import TYPE_CHECKING
+
+import torch
+from torch import Tensor, nn
+
+from nestor_amd import ops
+from nestor_amd.dispatch import GROUPED_MM_ALIGN, DispatchPlan, dispatch_plan
+from nestor_amd.expert_kernels import (
+    bank_is_fusable,
+    cat_cast,
+    combine_rows,
+    dispatch_rows,
+    swiglu,
+    swiglu_fused,
+)
+
+if TYPE_CHECKING:  # pragma: no cover
+    from nestor_amd.bank import StackedExpertBank
+
+__all__ = [
+    "GROUPED_MM_ALIGN",
+    "autocast_dtype",
+    "segment_mm",
+    "grouped_expert_rows",
+    "grouped_expert_combine",
+]
+
+
+def autocast_dtype(x: Tensor) -> torch.dtype:
+    """The dtype ``F.linear`` would compute in for ``x`` right now: the autocast
+    dtype of its device type when autocast is on, else ``x.dtype``
+    (nestor/backbones/grouped_mm.py:64-80)."""
+
+    kind = x.device.type
+    if torch.is_autocast_enabled(kind):
+        return torch.get_autocast_dtype(kind)
+    return x.dtype
+
+
+def _gemm_dtype(x: Tensor) -> torch.dtype:
+    dtype = autocast_dtype(x)
+    if dtype != torch.bfloat16:
+        raise NotImplementedError(
+            "the HIP expert path computes in bfloat16: run it under "
+            f"torch.autocast('cuda', torch.bfloat16) or pass bf16 inputs (got {dtype})"
+        )
+    return dtype
+
+
+def segment_mm(a: Tensor, b: Tensor, offs: Tensor) -> Tensor:
+    """Rows ``[offs[i-1], offs[i])`` of ``a`` through ``b[i]``; ``offs[-1]`` must
+    equal ``a.shape[0]``.  Differentiable in ``a`` and ``b``."""
+
+    table = ops.tile_schedule(offs, a.shape[0])
+    return ops.grouped_mm_op(a, b, table, offs, None, None)
+
+
+def _plan_mm(a: Tensor, b: Tensor, plan: DispatchPlan) -> Tensor:
+    """``segment_mm`` driven by a plan: its tile table skips the slack tail and
+    the weight gradient contracts over real rows only."""
+
+    return ops.grouped_mm_op(a, b, plan.tile_table, plan.offs, plan.padded_starts, plan.counts)
+
+
+def _bank_weights(
+    experts: Sequence[nn.Module], stacked: "StackedExpertBank | None", dtype: torch.dtype,
+    gated: bool,
+) -> tuple[Tensor, Tensor | None, Tensor]:
+    """(w_up, w_gate, w_down) as ``[E, d_in, h]`` / ``[E, h, d_out]`` in ``dtype``."""
+
+    if stacked is not None:
+        return stacked.cast(dtype)
+
+    def stack(mods: list[nn.Module]) -> Tensor:
+        return torch.stack([m.weight for m in mods]).to(dtype).transpose(-2, -1).contiguous()
+
+    w_up = stack([e.layers[0] for e in experts])
+    w_down = stack([e.layers[1] for e in experts])
+    w_gate = stack([e.gate for e in experts]) if gated else None
+    return w_up, w_gate, w_down
+
+
+def _row_bias(bias_bank: Tensor, index: Tensor, valid: Tensor | None) -> Tensor:
+    rows = bias_bank.index_select(0, index)
+    return rows if valid is None else rows * valid.unsqueeze(1)
+
+
+def _expert_rows_padded(
+    x: Tensor, experts: Sequence[nn.Module], plan: DispatchPlan, slots: int,
+    dtype: torch.dtype, *, fused_gate: bool, stacked: "StackedExpertBank | None",
+    hip_fused: bool, hip_cat_cast: bool = True,
+) -> Tensor:
+    """Dispatch, run the bank, return the PADDED down-projection rows
+    (nestor/backbones/grouped_mm.py:324-450)."""
+
+    first = experts[0]
+    gated = bool(getattr(first, "gated", False))
+    biased = first.layers[0].bias is not None
+    w_up, w_gate, w_down = _bank_weights(experts, stacked, dtype, gated)
+    x_pad = dispatch_rows(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots, dtype)
+
+    if hip_fused and gated and not biased:
+        # Both stacked banks read in place; SwiGLU in the GEMM epilogue.
+        _up_gate, hidden = ops.upgate_swiglu_op(
+            x_pad, w_up, w_gate, plan.tile_table, plan.offs, plan.padded_starts, plan.counts
+        )
+        return _plan_mm(hidden, w_down, plan)
+
+    gate_rows: Tensor | None = None
+    if gated and fused_gate and not biased:
+        if stacked is not None and hip_cat_cast and stacked.w_up.dtype == torch.float32:
+            w_up_gate = cat_cast(stacked.w_up, stacked.w_gate, dtype)
+        else:
+            w_up_gate = torch.cat([w_up, w_gate], dim=-1)
+        up_gate = _plan_mm(x_pad, w_up_gate, plan)
+        return _plan_mm(swiglu_fused(up_gate, w_up.shape[-1]), w_down, plan)
+
+    hidden = _plan_mm(x_pad, w_up, plan)
+    if biased:
+        b_up = (
+            stacked.b_up.to(dtype) if stacked is not None
+            else torch.stack([e.layers[0].bias for e in experts]).to(dtype)
+        )
+        hidden = hidden + _row_bias(b_up, plan.eid_pad, plan.pad_valid)
+    if gated:
+        gate_rows = _plan_mm(x_pad, w_gate, plan)
+        hidden = swiglu(hidden, gate_rows) if first.activation == "silu" else (
+            first._activation_fn(gate_rows) * hidden
+        )
+    else:
+        hidden = first._activation_fn(hidden)
+    return _plan_mm(hidden, w_down, plan)
+
+
+def grouped_expert_rows(
+    x: Tensor, experts: Sequence[nn.Module], expert_ids: Tensor, *,
+    fused_gate: bool = False, stacked: "StackedExpertBank | None" = None,
+    triton_index: bool = False,
+) -> Tensor:
+    """Row ``token * slots + slot`` of the result is
+    ``experts[expert_ids[token, slot]](x[token])``, unweighted, in the GEMM dtype.
+
+    ``triton_index`` is accepted for signature compatibility; the HIP index
+    build is the only one here.
+    """
+
+    del triton_index
+    num_tokens, slots = expert_ids.shape
+    dtype = _gemm_dtype(x)
+    flat_ids = expert_ids.reshape(-1)
+    plan = dispatch_plan(flat_ids, len(experts), slots, dtype)
+    out_pad = _expert_rows_padded(
+        x, experts, plan, slots, dtype, fused_gate=fused_gate, stacked=stacked, hip_fused=False
+    )
+    routed = _PaddedRowGather.apply(out_pad, plan.row_dest, plan.pad_src_row, plan.pad_valid)
+    if experts[0].layers[1].bias is not None:
+        b_down = (
+            stacked.b_down.to(dtype) if stacked is not None
+            else torch.stack([e.layers[1].bias for e in experts]).to(dtype)
+        )
+        routed = routed + _row_bias(b_down, flat_ids, None)
+    return routed
+
+
+class _PaddedRowGather(torch.autograd.Function):
+    """``y_pad[row_dest]`` whose backward is the gather at ``pad_src_row`` masked by
+    validity, never an atomic scatter (nestor/backbones/grouped_mm.py:134-156)."""
+
+    @staticmethod
+    def forward(ctx, y_pad, row_dest, pad_src_row, pad_valid):
+        ctx.save_for_backward(pad_src_row, pad_valid)
+        return y_pad.index_select(0, row_dest)
+
+    @staticmethod
+    def backward(ctx, grad_rows):
+        pad_src_row, pad_valid = ctx.saved_tensors
+        grad_pad = grad_rows.index_select(0, pad_src_row) * pad_valid.unsqueeze(1)
+        return grad_pad.to(pad_valid.dtype), None, None, None
+
+
+def grouped_expert_combine(
+    x: Tensor, experts: Sequence[nn.Module], expert_ids: Tensor, weights: Tensor, group: int,
+    *, fused_gate: bool = False, stacked: "StackedExpertBank | None" = None,
+    triton_index: bool = False, triton_fused: bool = False, triton_cat_cast: bool = True,
+    capacity: int = 0,
+) -> Tensor:
+    """``grouped_expert_rows`` weighted and summed over groups of ``group``
+    consecutive slots: ``[num_tokens, slots // group, d_out]`` in ``x``'s dtype.
+
+    ``triton_fused`` selects the fused HIP bank (bias-free SwiGLU only; other
+    banks take the composed kernels and the eager weighting).  ``capacity > 0``
+    is this implementation's extension: rows beyond a bank's capacity are
+    dropped in stable order and contribute exactly zero.
+    """
+
+    del triton_index
+    num_tokens, slots = expert_ids.shape
+    assert slots % group == 0, "group must divide the slot count"
+    fusable = bank_is_fusable(list(experts), fused_gate)
+    if not fusable:
+        if capacity > 0:
+            raise NotImplementedError("capacity limits need a bias-free SwiGLU bank")
+        rows = grouped_expert_rows(x, experts, expert_ids, fused_gate=fused_gate, stacked=stacked)
+        weighted = (rows * weights.reshape(-1, 1)).to(x.dtype)
+        return weighted.view(num_tokens, slots // group, group, -1).sum(2)
+
+    dtype = _gemm_dtype(x)
+    plan = dispatch_plan(expert_ids.reshape(-1), len(experts), slots, dtype, capacity)
+    out_pad = _expert_rows_padded(
+        x, experts, plan, slots, dtype, fused_gate=fused_gate, stacked=stacked,
+        hip_fused=triton_fused, hip_cat_cast=triton_cat_cast,
+    )
+    flat_w = weights.reshape(-1)
+    if capacity > 0:
+        flat_w = flat_w * plan.row_kept.to(flat_w.dtype)
+    combined = combine_rows(
+        out_pad, plan.row_dest, plan.pad_src_row, plan.pad_valid, flat_w, group, x.dtype
+    )
+    return combined.view(num_tokens, slots // group, -1)

@@ -1,0 +1,749 @@
+"""``torch.library`` custom ops (namespace ``nestor_hip``) over the C ABI.
+
+Each op allocates its outputs with torch, passes raw device pointers and the
+current HIP stream to ``libnestor_hip.so`` and returns; none reads device memory
+on the host, so a forward+backward enqueues without a single synchronisation.
+Every op has a fake (meta) kernel, and the differentiable ones register their
+backward as further custom ops, so the path traces under ``torch.compile``.
+
+Ops only exist for CUDA/HIP tensors: calling one with CPU tensors raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+from torch import Tensor
+
+from nestor_amd import _lib
+
+_NS = "nestor_hip"
+
+
+def _ptr(t: Tensor | None) -> ctypes.c_void_p | None:
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(t: Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _lib.F32
+    if dtype == torch.bfloat16:
+        return _lib.BF16
+    raise TypeError(f"nestor_hip kernels take float32 or bfloat16 here, got {dtype}")
+
+
+def _bf16(t: Tensor, name: str) -> Tensor:
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be bfloat16 (the GEMM dtype of the HIP path), got {t.dtype}")
+    return t.contiguous()
+
+
+def rows_pad_for(rows: int, num_banks: int) -> int:
+    a = _lib.ROW_ALIGN
+    return ((rows + a - 1) // a) * a + a * num_banks
+
+
+def max_tiles_for(rows_pad: int, num_banks: int) -> int:
+    return rows_pad // _lib.TILE_M + num_banks + 2
+
+
+# --------------------------------------------------------------------------
+# Index build
+# --------------------------------------------------------------------------
+@torch.library.custom_op(f"{_NS}::index_build", mutates_args=(), device_types="cuda")
+def index_build(
+    expert_ids: Tensor, num_banks: int, slots: int, capacity: int, valid_dtype: torch.dtype
+) -> list[Tensor]:
+    """[order, counts, raw_starts, padded_starts, offs, row_dest, pad_token,
+    pad_src_row, eid_pad, pad_valid, row_kept, tile_table]."""
+
+    ids = expert_ids.contiguous()
+    assert ids.dtype == torch.long and ids.dim() == 1
+    rows = ids.shape[0]
+    dev = ids.device
+    rows_pad = rows_pad_for(rows, num_banks)
+    max_tiles = max_tiles_for(rows_pad, num_banks)
+    i64 = dict(dtype=torch.long, device=dev)
+    order = torch.empty(rows, **i64)
+    counts = torch.empty(num_banks, **i64)
+    raw_starts = torch.empty(num_banks, **i64)
+    padded_starts = torch.empty(num_banks, **i64)
+    offs = torch.empty(num_banks, dtype=torch.int32, device=dev)
+    row_dest = torch.empty(rows, **i64)
+    pad_token = torch.empty(rows_pad, **i64)
+    pad_src_row = torch.empty(rows_pad, **i64)
+    eid_pad = torch.empty(rows_pad, **i64)
+    pad_valid = torch.empty(rows_pad, dtype=valid_dtype, device=dev)
+    row_kept = torch.empty(rows, dtype=torch.uint8, device=dev)
+    tile_table = torch.empty(3 * max_tiles + 1, dtype=torch.int32, device=dev)
+    ws_bytes = _lib.load().nestor_hip_index_build_workspace_bytes(rows, num_banks)
+    workspace = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+    _lib.call(
+        "nestor_hip_index_build", _ptr(ids), rows, num_banks, slots, rows_pad, capacity,
+        _code(valid_dtype), _ptr(order), _ptr(counts), _ptr(raw_starts), _ptr(padded_starts),
+        _ptr(offs), _ptr(row_dest), _ptr(pad_token), _ptr(pad_src_row), _ptr(eid_pad),
+        _ptr(pad_valid), _ptr(row_kept), _ptr(tile_table), max_tiles, _ptr(workspace),
+        workspace.numel(), _stream(ids),
+    )
+    return [order, counts, raw_starts, padded_starts, offs, row_dest, pad_token,
+            pad_src_row, eid_pad, pad_valid, row_kept, tile_table]
+
+
+@index_build.register_fake
+def _(expert_ids, num_banks, slots, capacity, valid_dtype):
+    rows = expert_ids.shape[0]
+    rows_pad = rows_pad_for(rows, num_banks)
+    max_tiles = max_tiles_for(rows_pad, num_banks)
+    new = expert_ids.new_empty
+    return [
+        new(rows), new(num_banks), new(num_banks), new(num_banks),
+        new(num_banks, dtype=torch.int32), new(rows), new(rows_pad), new(rows_pad),
+        new(rows_pad), new(rows_pad, dtype=valid_dtype), new(rows, dtype=torch.uint8),
+        new(3 * max_tiles + 1, dtype=torch.int32),
+    ]
+
+
+@torch.library.custom_op(f"{_NS}::build_dispatch_maps", mutates_args=(), device_types="cuda")
+def build_dispatch_maps_op(
+    expert_ids: Tensor, order: Tensor, padded_starts: Tensor, raw_starts: Tensor,
+    slots: int, rows_pad: int, valid_dtype: torch.dtype,
+) -> list[Tensor]:
+    ids = expert_ids.contiguous()
+    order = order.contiguous()
+    padded_starts = padded_starts.contiguous()
+    raw_starts = raw_starts.contiguous()
+    rows = order.shape[0]
+    dev = order.device
+    num_banks = padded_starts.shape[0]
+    row_dest = torch.empty(rows, dtype=torch.long, device=dev)
+    pad_token = torch.empty(rows_pad, dtype=torch.long, device=dev)
+    pad_src_row = torch.empty(rows_pad, dtype=torch.long, device=dev)
+    eid_pad = torch.empty(rows_pad, dtype=torch.long, device=dev)
+    pad_valid = torch.empty(rows_pad, dtype=valid_dtype, device=dev)
+    _lib.call(
+        "nestor_hip_build_dispatch_maps", _ptr(ids), _ptr(order), _ptr(padded_starts),
+        _ptr(raw_starts), rows, num_banks, slots, rows_pad, _code(valid_dtype),
+        _ptr(row_dest), _ptr(pad_token), _ptr(pad_src_row), _ptr(eid_pad), _ptr(pad_valid),
+        _stream(order),
+    )
+    return [row_dest, pad_token, pad_src_row, eid_pad, pad_valid]
+
+
+@build_dispatch_maps_op.register_fake
+def _(expert_ids, order, padded_starts, raw_starts, slots, rows_pad, valid_dtype):
+    rows = order.shape[0]
+    new = order.new_empty
+    return [new(rows), new(rows_pad), new(rows_pad), new(rows_pad),
+            new(rows_pad, dtype=valid_dtype)]
+
+
+@torch.library.custom_op(f"{_NS}::tile_schedule", mutates_args=(), device_types="cuda")
+def tile_schedule(offs: Tensor, rows_pad: int) -> Tensor:
+    offs = offs.contiguous()
+    assert offs.dtype == torch.int32
+    num_banks = offs.shape[0]
+    max_tiles = max_tiles_for(rows_pad, num_banks)
+    table = torch.empty(3 * max_tiles + 1, dtype=torch.int32, device=offs.device)
+    _lib.call("nestor_hip_tile_schedule", _ptr(offs), num_banks, _ptr(table), max_tiles,
+              _stream(offs))
+    return table
+
+
+@tile_schedule.register_fake
+def _(offs, rows_pad):
+    return offs.new_empty(3 * max_tiles_for(rows_pad, offs.shape[0]) + 1)
+
+
+def _table_max_tiles(tile_table: Tensor) -> int:
+    return (tile_table.shape[0] - 1) // 3
+
+
+# --------------------------------------------------------------------------
+# Row moves
+# --------------------------------------------------------------------------
+@torch.library.custom_op(f"{_NS}::dispatch_rows_fwd", mutates_args=(), device_types="cuda")
+def dispatch_rows_fwd(x: Tensor, pad_token: Tensor, pad_valid: Tensor) -> Tensor:
+    x = x.contiguous()
+    rows_pad = pad_token.shape[0]
+    out = torch.empty(rows_pad, x.shape[1], dtype=torch.bfloat16, device=x.device)
+    _lib.call(
+        "nestor_hip_dispatch_rows_fwd", _ptr(x), _code(x.dtype), _ptr(pad_token.contiguous()),
+        _ptr(pad_valid.contiguous()), _code(pad_valid.dtype), _ptr(out), rows_pad,
+        x.shape[1], _stream(x),
+    )
+    return out
+
+
+@dispatch_rows_fwd.register_fake
+def _(x, pad_token, pad_valid):
+    return x.new_empty(pad_token.shape[0], x.shape[1], dtype=torch.bfloat16)
+
+
+@torch.library.custom_op(f"{_NS}::dispatch_rows_bwd", mutates_args=(), device_types="cuda")
+def dispatch_rows_bwd(
+    grad_pad: Tensor, row_dest: Tensor, num_tokens: int, slots: int, x_dtype: torch.dtype
+) -> Tensor:
+    grad_pad = _bf16(grad_pad, "grad_pad")
+    dim = grad_pad.shape[1]
+    out = torch.empty(num_tokens, dim, dtype=x_dtype, device=grad_pad.device)
+    _lib.call(
+        "nestor_hip_dispatch_rows_bwd", _ptr(grad_pad), _ptr(row_dest.contiguous()), _ptr(out),
+        _code(x_dtype), num_tokens, slots, dim, _stream(grad_pad),
+    )
+    return out
+
+
+@dispatch_rows_bwd.register_fake
+def _(grad_pad, row_dest, num_tokens, slots, x_dtype):
+    return grad_pad.new_empty(num_tokens, grad_pad.shape[1], dtype=x_dtype)
+
+
+@torch.library.custom_op(f"{_NS}::dispatch_rows", mutates_args=(), device_types="cuda")
+def dispatch_rows_op(
+    x: Tensor, pad_token: Tensor, pad_valid: Tensor, row_dest: Tensor, slots: int
+) -> Tensor:
+    return dispatch_rows_fwd(x, pad_token, pad_valid)
+
+
+@dispatch_rows_op.register_fake
+def _(x, pad_token, pad_valid, row_dest, slots):
+    return x.new_empty(pad_token.shape[0], x.shape[1], dtype=torch.bfloat16)
+
+
+def _dispatch_setup(ctx, inputs, output):
+    x, _pad_token, _pad_valid, row_dest, slots = inputs
+    ctx.save_for_backward(row_dest)
+    ctx.slots = slots
+    ctx.num_tokens = x.shape[0]
+    ctx.x_dtype = x.dtype
+
+
+def _dispatch_backward(ctx, grad_pad):
+    (row_dest,) = ctx.saved_tensors
+    gx = dispatch_rows_bwd(grad_pad, row_dest, ctx.num_tokens, ctx.slots, ctx.x_dtype)
+    return gx, None, None, None, None
+
+
+dispatch_rows_op.register_autograd(_dispatch_backward, setup_context=_dispatch_setup)
+
+
+@torch.library.custom_op(f"{_NS}::swiglu_fwd", mutates_args=(), device_types="cuda")
+def swiglu_fwd(up_gate: Tensor, hidden: int) -> Tensor:
+    """``up_gate`` is ``[rows, 2*hidden]`` (up | gate)."""
+
+    up_gate = _bf16(up_gate, "up_gate")
+    rows = up_gate.shape[0]
+    out = torch.empty(rows, hidden, dtype=torch.bfloat16, device=up_gate.device)
+    base = up_gate.data_ptr()
+    _lib.call(
+        "nestor_hip_swiglu_fwd", ctypes.c_void_p(base), ctypes.c_void_p(base + 2 * hidden),
+        _ptr(out), rows, hidden, 2 * hidden, hidden, _stream(up_gate),
+    )
+    return out
+
+
+@swiglu_fwd.register_fake
+def _(up_gate, hidden):
+    return up_gate.new_empty(up_gate.shape[0], hidden)
+
+
+@torch.library.custom_op(f"{_NS}::swiglu_bwd", mutates_args=(), device_types="cuda")
+def swiglu_bwd(grad_out: Tensor, up_gate: Tensor, hidden: int) -> Tensor:
+    grad_out = _bf16(grad_out, "grad_out")
+    up_gate = _bf16(up_gate, "up_gate")
+    rows = up_gate.shape[0]
+    grad = torch.empty_like(up_gate)
+    base = up_gate.data_ptr()
+    gbase = grad.data_ptr()
+    _lib.call(
+        "nestor_hip_swiglu_bwd", _ptr(grad_out), ctypes.c_void_p(base),
+        ctypes.c_void_p(base + 2 * hidden), ctypes.c_void_p(gbase),
+        ctypes.c_void_p(gbase + 2 * hidden), rows, hidden, 2 * hidden, 2 * hidden, hidden,
+        _stream(up_gate),
+    )
+    return grad
+
+
+@swiglu_bwd.register_fake
+def _(grad_out, up_gate, hidden):
+    return torch.empty_like(up_gate)
+
+
+@torch.library.custom_op(f"{_NS}::swiglu_fused", mutates_args=(), device_types="cuda")
+def swiglu_fused_op(up_gate: Tensor, hidden: int) -> Tensor:
+    return swiglu_fwd(up_gate, hidden)
+
+
+@swiglu_fused_op.register_fake
+def _(up_gate, hidden):
+    return up_gate.new_empty(up_gate.shape[0], hidden)
+
+
+def _swiglu_fused_setup(ctx, inputs, output):
+    up_gate, hidden = inputs
+    ctx.save_for_backward(up_gate)
+    ctx.hidden = hidden
+
+
+def _swiglu_fused_backward(ctx, grad_out):
+    (up_gate,) = ctx.saved_tensors
+    return swiglu_bwd(grad_out, up_gate, ctx.hidden), None
+
+
+swiglu_fused_op.register_autograd(_swiglu_fused_backward, setup_context=_swiglu_fused_setup)
+
+
+@torch.library.custom_op(f"{_NS}::swiglu_split_fwd", mutates_args=(), device_types="cuda")
+def swiglu_split_fwd(up: Tensor, gate: Tensor) -> Tensor:
+    up = _bf16(up, "up")
+    gate = _bf16(gate, "gate")
+    rows, hidden = up.shape
+    out = torch.empty_like(up)
+    _lib.call("nestor_hip_swiglu_fwd", _ptr(up), _ptr(gate), _ptr(out), rows, hidden, hidden,
+              hidden, _stream(up))
+    return out
+
+
+@swiglu_split_fwd.register_fake
+def _(up, gate):
+    return torch.empty_like(up)
+
+
+@torch.library.custom_op(f"{_NS}::swiglu_split_bwd", mutates_args=(), device_types="cuda")
+def swiglu_split_bwd(grad_out: Tensor, up: Tensor, gate: Tensor) -> list[Tensor]:
+    grad_out = _bf16(grad_out, "grad_out")
+    up = _bf16(up, "up")
+    gate = _bf16(gate, "gate")
+    rows, hidden = up.shape
+    gup = torch.empty_like(up)
+    ggate = torch.empty_like(gate)
+    _lib.call(
+        "nestor_hip_swiglu_bwd", _ptr(grad_out), _ptr(up), _ptr(gate), _ptr(gup), _ptr(ggate),
+        rows, hidden, hidden, hidden, hidden, _stream(up),
+    )
+    return [gup, ggate]
+
+
+@swiglu_split_bwd.register_fake
+def _(grad_out, up, gate):
+    return [torch.empty_like(up), torch.empty_like(gate)]
+
+
+@torch.library.custom_op(f"{_NS}::swiglu", mutates_args=(), device_types="cuda")
+def swiglu_op(up: Tensor, gate: Tensor) -> Tensor:
+    return swiglu_split_fwd(up, gate)
+
+
+@swiglu_op.register_fake
+def _(up, gate):
+    return torch.empty_like(up)
+
+
+def _swiglu_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs)
+
+
+def _swiglu_backward(ctx, grad_out):
+    up, gate = ctx.saved_tensors
+    gup, ggate = swiglu_split_bwd(grad_out, up, gate)
+    return gup, ggate
+
+
+swiglu_op.register_autograd(_swiglu_backward, setup_context=_swiglu_setup)
+
+
+@torch.library.custom_op(f"{_NS}::cat_cast_fwd", mutates_args=(), device_types="cuda")
+def cat_cast_fwd(a: Tensor, b: Tensor) -> Tensor:
+    a = a.contiguous()
+    b = b.contiguous()
+    assert a.dtype == torch.float32 and b.dtype == torch.float32
+    hidden = a.shape[-1]
+    rows = a.numel() // hidden
+    out = torch.empty(*a.shape[:-1], 2 * hidden, dtype=torch.bfloat16, device=a.device)
+    _lib.call("nestor_hip_cat_cast_fwd", _ptr(a), _ptr(b), _ptr(out), rows, hidden, _stream(a))
+    return out
+
+
+@cat_cast_fwd.register_fake
+def _(a, b):
+    return a.new_empty(*a.shape[:-1], 2 * a.shape[-1], dtype=torch.bfloat16)
+
+
+@torch.library.custom_op(f"{_NS}::cat_cast_bwd", mutates_args=(), device_types="cuda")
+def cat_cast_bwd(grad: Tensor) -> list[Tensor]:
+    grad = _bf16(grad, "grad")
+    hidden = grad.shape[-1] // 2
+    rows = grad.numel() // (2 * hidden)
+    shape = (*grad.shape[:-1], hidden)
+    ga = torch.empty(shape, dtype=torch.float32, device=grad.device)
+    gb = torch.empty(shape, dtype=torch.float32, device=grad.device)
+    _lib.call("nestor_hip_cat_cast_bwd", _ptr(grad), _ptr(ga), _ptr(gb), rows, hidden,
+              _stream(grad))
+    return [ga, gb]
+
+
+@cat_cast_bwd.register_fake
+def _(grad):
+    shape = (*grad.shape[:-1], grad.shape[-1] // 2)
+    return [grad.new_empty(shape, dtype=torch.float32), grad.new_empty(shape, dtype=torch.float32)]
+
+
+@torch.library.custom_op(f"{_NS}::cat_cast", mutates_args=(), device_types="cuda")
+def cat_cast_op(a: Tensor, b: Tensor) -> Tensor:
+    return cat_cast_fwd(a, b)
+
+
+@cat_cast_op.register_fake
+def _(a, b):
+    return a.new_empty(*a.shape[:-1], 2 * a.shape[-1], dtype=torch.bfloat16)
+
+
+def _cat_cast_backward(ctx, grad):
+    ga, gb = cat_cast_bwd(grad)
+    return ga, gb
+
+
+cat_cast_op.register_autograd(_cat_cast_backward)
+
+
+@torch.library.custom_op(f"{_NS}::combine_rows_fwd", mutates_args=(), device_types="cuda")
+def combine_rows_fwd(
+    y_pad: Tensor, row_dest: Tensor, weights: Tensor, group: int, out_dtype: torch.dtype,
+    round_term: bool,
+) -> Tensor:
+    y_pad = _bf16(y_pad, "y_pad")
+    weights = weights.contiguous()
+    rows = row_dest.shape[0]
+    n_out = rows // group
+    dim = y_pad.shape[1]
+    out = torch.empty(n_out, dim, dtype=out_dtype, device=y_pad.device)
+    _lib.call(
+        "nestor_hip_combine_rows_fwd", _ptr(y_pad), _ptr(row_dest.contiguous()), _ptr(weights),
+        _code(weights.dtype), _ptr(out), _code(out_dtype), n_out, group, dim,
+        1 if round_term else 0, _stream(y_pad),
+    )
+    return out
+
+
+@combine_rows_fwd.register_fake
+def _(y_pad, row_dest, weights, group, out_dtype, round_term):
+    return y_pad.new_empty(row_dest.shape[0] // group, y_pad.shape[1], dtype=out_dtype)
+
+
+@torch.library.custom_op(f"{_NS}::combine_rows_bwd", mutates_args=(), device_types="cuda")
+def combine_rows_bwd(
+    grad_out: Tensor, y_pad: Tensor, pad_src_row: Tensor, pad_valid: Tensor, weights: Tensor,
+    group: int, need_w: bool,
+) -> list[Tensor]:
+    grad_out = grad_out.contiguous()
+    y_pad = _bf16(y_pad, "y_pad")
+    weights = weights.contiguous()
+    rows_pad, dim = y_pad.shape
+    grad_y = torch.empty_like(y_pad)
+    # Rows that own no padded slot (dropped by a capacity limit) keep gradient 0.
+    grad_w = torch.zeros(weights.shape[0], dtype=torch.float32, device=y_pad.device)
+    _lib.call(
+        "nestor_hip_combine_rows_bwd", _ptr(grad_out), _code(grad_out.dtype), _ptr(y_pad),
+        _ptr(pad_src_row.contiguous()), _ptr(pad_valid.contiguous()), _code(pad_valid.dtype),
+        _ptr(weights), _code(weights.dtype), _ptr(grad_y), _ptr(grad_w) if need_w else None,
+        rows_pad, group, dim, _stream(y_pad),
+    )
+    return [grad_y, grad_w]
+
+
+@combine_rows_bwd.register_fake
+def _(grad_out, y_pad, pad_src_row, pad_valid, weights, group, need_w):
+    return [torch.empty_like(y_pad), y_pad.new_empty(weights.shape[0], dtype=torch.float32)]
+
+
+@torch.library.custom_op(f"{_NS}::combine_rows", mutates_args=(), device_types="cuda")
+def combine_rows_op(
+    y_pad: Tensor, row_dest: Tensor, pad_src_row: Tensor, pad_valid: Tensor, weights: Tensor,
+    group: int, out_dtype: torch.dtype,
+) -> Tensor:
+    promoted = torch.promote_types(y_pad.dtype, weights.dtype)
+    round_term = promoted != torch.float32 or out_dtype != torch.float32
+    return combine_rows_fwd(y_pad, row_dest, weights, group, out_dtype, round_term)
+
+
+@combine_rows_op.register_fake
+def _(y_pad, row_dest, pad_src_row, pad_valid, weights, group, out_dtype):
+    return y_pad.new_empty(row_dest.shape[0] // group, y_pad.shape[1], dtype=out_dtype)
+
+
+def _combine_setup(ctx, inputs, output):
+    y_pad, _row_dest, pad_src_row, pad_valid, weights, group, _out_dtype = inputs
+    ctx.save_for_backward(y_pad, pad_src_row, pad_valid, weights)
+    ctx.group = group
+
+
+def _combine_backward(ctx, grad_out):
+    y_pad, pad_src_row, pad_valid, weights = ctx.saved_tensors
+    need_w = ctx.needs_input_grad[4]
+    grad_y, grad_w = combine_rows_bwd(
+        grad_out, y_pad, pad_src_row, pad_valid, weights, ctx.group, need_w
+    )
+    return grad_y, None, None, None, grad_w.to(weights.dtype) if need_w else None, None, None
+
+
+combine_rows_op.register_autograd(_combine_backward, setup_context=_combine_setup)
+
+
+# --------------------------------------------------------------------------
+# Grouped GEMMs
+# --------------------------------------------------------------------------
+@torch.library.custom_op(f"{_NS}::grouped_gemm_nn", mutates_args=(), device_types="cuda")
+def grouped_gemm_nn(a: Tensor, b: Tensor, tile_table: Tensor) -> Tensor:
+    a = _bf16(a, "a")
+    b = _bf16(b, "b")
+    rows_pad, k = a.shape
+    num_banks, kb, n = b.shape
+    assert kb == k
+    out = torch.empty(rows_pad, n, dtype=torch.bfloat16, device=a.device)
+    _lib.call(
+        "nestor_hip_grouped_gemm_nn", _ptr(a), _ptr(b), _ptr(out), rows_pad, k, n, num_banks,
+        _ptr(tile_table), _table_max_tiles(tile_table), _stream(a),
+    )
+    return out
+
+
+@grouped_gemm_nn.register_fake
+def _(a, b, tile_table):
+    return a.new_empty(a.shape[0], b.shape[2])
+
+
+@torch.library.custom_op(f"{_NS}::grouped_gemm_nt", mutates_args=(), device_types="cuda")
+def grouped_gemm_nt(a: Tensor, b: Tensor, tile_table: Tensor) -> Tensor:
+    """``a [rows, K] @ b[bank]^T`` with ``b [E, N, K]``."""
+
+    a = _bf16(a, "a")
+    b = _bf16(b, "b")
+    rows_pad, k = a.shape
+    num_banks, n, kb = b.shape
+    assert kb == k
+    out = torch.empty(rows_pad, n, dtype=torch.bfloat16, device=a.device)
+    _lib.call(
+        "nestor_hip_grouped_gemm_nt", _ptr(a), _ptr(b), _ptr(out), rows_pad, k, n, num_banks,
+        _ptr(tile_table), _table_max_tiles(tile_table), _stream(a),
+    )
+    return out
+
+
+@grouped_gemm_nt.register_fake
+def _(a, b, tile_table):
+    return a.new_empty(a.shape[0], b.shape[1])
+
+
+@torch.library.custom_op(f"{_NS}::grouped_gemm_tn", mutates_args=(), device_types="cuda")
+def grouped_gemm_tn(
+    a: Tensor, g: Tensor, offs: Tensor, seg_start: Tensor | None, seg_count: Tensor | None
+) -> Tensor:
+    """``out[e] = a[seg e]^T @ g[seg e]`` -> ``[E, M, N]`` bf16.  ``a`` / ``g`` may be
+    column slices of wider row-major tensors (unit inner stride)."""
+
+    assert a.dtype == torch.bfloat16 and g.dtype == torch.bfloat16
+    assert a.stride(1) == 1 and g.stride(1) == 1
+    rows_pad, m = a.shape
+    n = g.shape[1]
+    num_banks = offs.shape[0]
+    out = torch.empty(num_banks, m, n, dtype=torch.bfloat16, device=a.device)
+    _lib.call(
+        "nestor_hip_grouped_gemm_tn", _ptr(a), a.stride(0), _ptr(g), g.stride(0), _ptr(out), n,
+        m * n, rows_pad, m, n, num_banks, _ptr(offs.contiguous()), _ptr(seg_start),
+        _ptr(seg_count), _stream(a),
+    )
+    return out
+
+
+@grouped_gemm_tn.register_fake
+def _(a, g, offs, seg_start, seg_count):
+    return a.new_empty(offs.shape[0], a.shape[1], g.shape[1])
+
+
+@torch.library.custom_op(f"{_NS}::upgate_swiglu_fwd", mutates_args=(), device_types="cuda")
+def upgate_swiglu_fwd(
+    x_pad: Tensor, w_up: Tensor, w_gate: Tensor, tile_table: Tensor
+) -> list[Tensor]:
+    """[up_gate ``[rows_pad, 2H]``, hidden ``[rows_pad, H]``]."""
+
+    x_pad = _bf16(x_pad, "x_pad")
+    w_up = _bf16(w_up, "w_up")
+    w_gate = _bf16(w_gate, "w_gate")
+    rows_pad, k = x_pad.shape
+    num_banks, kb, h = w_up.shape
+    assert kb == k and w_gate.shape == w_up.shape
+    up_gate = torch.empty(rows_pad, 2 * h, dtype=torch.bfloat16, device=x_pad.device)
+    hidden = torch.empty(rows_pad, h, dtype=torch.bfloat16, device=x_pad.device)
+    _lib.call(
+        "nestor_hip_grouped_gemm_upgate_swiglu", _ptr(x_pad), _ptr(w_up), _ptr(w_gate),
+        _ptr(up_gate), _ptr(hidden), rows_pad, k, h, num_banks, _ptr(tile_table),
+        _table_max_tiles(tile_table), _stream(x_pad),
+    )
+    return [up_gate, hidden]
+
+
+@upgate_swiglu_fwd.register_fake
+def _(x_pad, w_up, w_gate, tile_table):
+    h = w_up.shape[2]
+    return [x_pad.new_empty(x_pad.shape[0], 2 * h), x_pad.new_empty(x_pad.shape[0], h)]
+
+
+@torch.library.custom_op(f"{_NS}::grouped_gemm_nt_upgate", mutates_args=(), device_types="cuda")
+def grouped_gemm_nt_upgate(
+    g_up_gate: Tensor, w_up: Tensor, w_gate: Tensor, tile_table: Tensor
+) -> Tensor:
+    g_up_gate = _bf16(g_up_gate, "g_up_gate")
+    w_up = _bf16(w_up, "w_up")
+    w_gate = _bf16(w_gate, "w_gate")
+    rows_pad = g_up_gate.shape[0]
+    num_banks, k, h = w_up.shape
+    out = torch.empty(rows_pad, k, dtype=torch.bfloat16, device=g_up_gate.device)
+    _lib.call(
+        "nestor_hip_grouped_gemm_nt_upgate", _ptr(g_up_gate), _ptr(w_up), _ptr(w_gate),
+        _ptr(out), rows_pad, k, h, num_banks, _ptr(tile_table), _table_max_tiles(tile_table),
+        _stream(g_up_gate),
+    )
+    return out
+
+
+@grouped_gemm_nt_upgate.register_fake
+def _(g_up_gate, w_up, w_gate, tile_table):
+    return g_up_gate.new_empty(g_up_gate.shape[0], w_up.shape[1])
+
+
+@torch.library.custom_op(f"{_NS}::grouped_gemm_fp8w_nn", mutates_args=(), device_types="cuda")
+def grouped_gemm_fp8w_nn(a: Tensor, b_q: Tensor, scale: Tensor, tile_table: Tensor) -> Tensor:
+    a = _bf16(a, "a")
+    b_q = b_q.contiguous()
+    scale = scale.contiguous()
+    assert b_q.dtype == torch.float8_e4m3fn and scale.dtype == torch.float32
+    rows_pad, k = a.shape
+    num_banks, kb, n = b_q.shape
+    assert kb == k and scale.shape == (num_banks, n)
+    out = torch.empty(rows_pad, n, dtype=torch.bfloat16, device=a.device)
+    _lib.call(
+        "nestor_hip_grouped_gemm_fp8w_nn", _ptr(a), _ptr(b_q), _ptr(scale), _ptr(out), rows_pad,
+        k, n, num_banks, _ptr(tile_table), _table_max_tiles(tile_table), _stream(a),
+    )
+    return out
+
+
+@grouped_gemm_fp8w_nn.register_fake
+def _(a, b_q, scale, tile_table):
+    return a.new_empty(a.shape[0], b_q.shape[2])
+
+
+# Differentiable grouped matmul: out = a @ b[bank] per segment.
+@torch.library.custom_op(f"{_NS}::grouped_mm", mutates_args=(), device_types="cuda")
+def grouped_mm_op(
+    a: Tensor, b: Tensor, tile_table: Tensor, offs: Tensor, seg_start: Tensor | None,
+    seg_count: Tensor | None,
+) -> Tensor:
+    return grouped_gemm_nn(a, b, tile_table)
+
+
+@grouped_mm_op.register_fake
+def _(a, b, tile_table, offs, seg_start, seg_count):
+    return a.new_empty(a.shape[0], b.shape[2])
+
+
+def _grouped_mm_setup(ctx, inputs, output):
+    a, b, tile_table, offs, seg_start, seg_count = inputs
+    ctx.save_for_backward(a, b, tile_table, offs, seg_start, seg_count)
+
+
+def _grouped_mm_backward(ctx, grad):
+    a, b, tile_table, offs, seg_start, seg_count = ctx.saved_tensors
+    grad = grad.contiguous()
+    ga = gb = None
+    if ctx.needs_input_grad[0]:
+        # b [E, K, N] read as [E, N', K'] with N' = K, K' = N: a @ b^T form.
+        ga = grouped_gemm_nt(grad, b, tile_table)
+    if ctx.needs_input_grad[1]:
+        gb = grouped_gemm_tn(a, grad, offs, seg_start, seg_count)
+    return ga, gb, None, None, None, None
+
+
+grouped_mm_op.register_autograd(_grouped_mm_backward, setup_context=_grouped_mm_setup)
+
+
+# Differentiable fused up|gate projection + SwiGLU.
+@torch.library.custom_op(f"{_NS}::upgate_swiglu", mutates_args=(), device_types="cuda")
+def upgate_swiglu_op(
+    x_pad: Tensor, w_up: Tensor, w_gate: Tensor, tile_table: Tensor, offs: Tensor,
+    seg_start: Tensor | None, seg_count: Tensor | None,
+) -> list[Tensor]:
+    return upgate_swiglu_fwd(x_pad, w_up, w_gate, tile_table)
+
+
+@upgate_swiglu_op.register_fake
+def _(x_pad, w_up, w_gate, tile_table, offs, seg_start, seg_count):
+    h = w_up.shape[2]
+    return [x_pad.new_empty(x_pad.shape[0], 2 * h), x_pad.new_empty(x_pad.shape[0], h)]
+
+
+def _upgate_setup(ctx, inputs, output):
+    x_pad, w_up, w_gate, tile_table, offs, seg_start, seg_count = inputs
+    up_gate, _hidden = output
+    ctx.save_for_backward(x_pad, w_up, w_gate, tile_table, offs, seg_start, seg_count, up_gate)
+    ctx.set_materialize_grads(False)
+
+
+def _upgate_backward(ctx, grads):
+    grad_up_gate, grad_hidden = grads
+    x_pad, w_up, w_gate, tile_table, offs, seg_start, seg_count, up_gate = ctx.saved_tensors
+    h = w_up.shape[2]
+    g = None
+    if grad_hidden is not None:
+        g = swiglu_bwd(grad_hidden.contiguous(), up_gate, h)
+    if grad_up_gate is not None:
+        g = grad_up_gate.contiguous() if g is None else g + grad_up_gate
+    if g is None:
+        return None, None, None, None, None, None, None
+    gx = gup = ggate = None
+    if ctx.needs_input_grad[0]:
+        gx = grouped_gemm_nt_upgate(g, w_up, w_gate, tile_table)
+    if ctx.needs_input_grad[1]:
+        gup = grouped_gemm_tn(x_pad, g[:, :h], offs, seg_start, seg_count)
+    if ctx.needs_input_grad[2]:
+        ggate = grouped_gemm_tn(x_pad, g[:, h:], offs, seg_start, seg_count)
+    return gx, gup, ggate, None, None, None, None
+
+
+upgate_swiglu_op.register_autograd(_upgate_backward, setup_context=_upgate_setup)
+
+
+# --------------------------------------------------------------------------
+# Router epilogue
+# --------------------------------------------------------------------------
+@torch.library.custom_op(f"{_NS}::router_topk", mutates_args=(), device_types="cuda")
+def router_topk(
+    scores: Tensor, choice_bias: Tensor, mask: Tensor | None, top_k: int, gate_mode: int
+) -> list[Tensor]:
+    """scores ``[n, C]``, choice_bias ``[rows_b, C]`` fp32 (row % rows_b), mask ``[n]``
+    bool/uint8 -> [softmax_probs fp32, topk_indices int64, gates (scores dtype)]."""
+
+    scores = scores.contiguous()
+    n, c = scores.shape
+    bias = choice_bias.contiguous().float().reshape(-1, c)
+    m = None if mask is None else mask.contiguous().view(torch.uint8)
+    probs = torch.empty(n, c, dtype=torch.float32, device=scores.device)
+    topk = torch.empty(n, top_k, dtype=torch.long, device=scores.device)
+    gates = torch.empty_like(scores)
+    _lib.call(
+        "nestor_hip_router_topk", _ptr(scores), _code(scores.dtype), _ptr(bias), bias.shape[0],
+        _ptr(m), _ptr(probs), _ptr(topk), _ptr(gates), n, c, top_k, gate_mode, _stream(scores),
+    )
+    return [probs, topk, gates]
+
+
+@router_topk.register_fake
+def _(scores, choice_bias, mask, top_k, gate_mode):
+    n, c = scores.shape
+    return [scores.new_empty(n, c, dtype=torch.float32),
+            scores.new_empty(n, top_k, dtype=torch.long), torch.empty_like(scores)]

@@ -1,0 +1,258 @@
+"""The hybrid public / column-private expert-pool MLP on the HIP path.
+
+Mirrors ``ExpertPoolMLP`` (nestor/backbones/expert_pools.py:110-1114): for each
+token
+
+    MLP(h) = a_pub  * sum_e public_gate_e * PublicExpert_e(h)
+           + a_priv * sum_g column_gate_g * sum_e private_gate_(g,e) * PrivateExpert_(g,e)(h)
+
+with ``(a_pub, a_priv) = softmax(path_gate(h))``.  The public pool is one bank
+call (``slots = k_p``), the ``G x Q`` private experts one flattened bank indexed
+``g * Q + e`` (``slots = k_a * k_q``).  Three output layouts: summed
+(``forward``), per column (``forward_per_group``) and per attention slot
+(``forward_per_slot``).
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from nestor_amd import flags
+from nestor_amd.bank import Linear2, StackedBanksMixin, SwigluExpert
+from nestor_amd.grouped import grouped_expert_combine
+from nestor_amd.router import Router, RouterOutput, check_batchable, route_private_batched
+
+
+def round_to_multiple_of_8(value: float) -> int:
+    """``max(8, round(value / 8) * 8)`` (nestor/backbones/expert_pool_dispatch.py:25-35)."""
+
+    return max(8, int(round(value / 8.0)) * 8)
+
+
+def public_expert_hidden_dim(dim: int, public_top_k: int, *, active_budget: float | None = None) -> int:
+    """``round8(budget * d / k_p)``, budget 2 by default (expert_pool_dispatch.py:38-62)."""
+
+    budget = 2.0 if active_budget is None else float(active_budget)
+    return round_to_multiple_of_8(budget * dim / public_top_k)
+
+
+def private_expert_hidden_dim(dim: int, num_groups_per_token: int, private_top_k: int, *,
+                              with_public_pool: bool = True,
+                              active_budget: float | None = None) -> int:
+    """``round8(budget * d / (k_a * k_q))``; budget 2 beside a public pool, 4 alone
+    (expert_pool_dispatch.py:65-105)."""
+
+    if active_budget is not None:
+        budget = float(active_budget)
+    else:
+        budget = 2.0 if with_public_pool else 4.0
+    return round_to_multiple_of_8(budget * dim / (num_groups_per_token * private_top_k))
+
+
+class ExpertPoolMLP(StackedBanksMixin, nn.Module):
+    """Public + column-private SwiGLU expert pools behind layer-local routers."""
+
+    def __init__(self, dim: int, num_groups: int, num_groups_per_token: int,
+                 num_public_experts: int, public_top_k: int, num_private_experts: int,
+                 private_top_k: int, router_score_mlp_hidden_dims: list[int],
+                 router_score_mlp_activation: str = "gelu",
+                 router_noise_mlp_hidden_dims: list[int] | None = None,
+                 router_noise_mlp_activation: str = "gelu", *,
+                 loss_free_balancing: bool = False, bias_update_rate: float = 0.0,
+                 active_budget: float | None = None, public_budget: float | None = None,
+                 private_gate_mode: str = "renorm") -> None:
+        super().__init__()
+        if num_private_experts < 1:
+            raise ValueError("ExpertPoolMLP requires a private pool: num_private_experts must be > 0.")
+        if not 1 <= num_groups_per_token <= num_groups:
+            raise ValueError("num_groups_per_token must be in [1, num_groups].")
+        self.dim = dim
+        self.num_groups = num_groups
+        self.num_groups_per_token = num_groups_per_token
+        self.num_public_experts = num_public_experts
+        self.public_top_k = public_top_k
+        self.num_private_experts = num_private_experts
+        self.private_top_k = private_top_k
+        self.private_gate_mode = private_gate_mode
+        self.has_public_pool = num_public_experts > 0
+        self.public_hidden_dim = (
+            public_expert_hidden_dim(dim, public_top_k, active_budget=public_budget)
+            if self.has_public_pool else 0
+        )
+        self.private_hidden_dim = private_expert_hidden_dim(
+            dim, num_groups_per_token, private_top_k,
+            with_public_pool=self.has_public_pool, active_budget=active_budget,
+        )
+
+        def make_router(choices: int, top_k: int, gate_mode: str = "renorm") -> Router:
+            return Router(dim, choices, top_k, router_score_mlp_hidden_dims,
+                          router_score_mlp_activation, loss_free_balancing=loss_free_balancing,
+                          bias_update_rate=bias_update_rate, gate_mode=gate_mode)
+
+        self.public_router = make_router(num_public_experts, public_top_k) if self.has_public_pool else None
+        self.private_routers = nn.ModuleList(
+            [make_router(num_private_experts, private_top_k, private_gate_mode) for _ in range(num_groups)]
+        )
+        self.public_experts = (
+            nn.ModuleList([SwigluExpert(dim, self.public_hidden_dim, dim) for _ in range(num_public_experts)])
+            if self.has_public_pool else None
+        )
+        self.private_experts = nn.ModuleList(
+            [nn.ModuleList([SwigluExpert(dim, self.private_hidden_dim, dim)
+                            for _ in range(num_private_experts)]) for _ in range(num_groups)]
+        )
+        if self.has_public_pool:
+            self.path_gate = Linear2(dim, 2, bias=False)
+            with torch.no_grad():
+                self.path_gate.weight.zero_()  # alpha = (0.5, 0.5) at step 0
+        else:
+            self.path_gate = None
+        self.grouped_dispatch = False if flags.pool_grouped_mm_disabled() else None
+        self.fused_gate = flags.fused_gate_requested()
+        self.triton_index = flags.triton_index_requested() and flags.triton_index_available()
+        self.triton_fused = flags.triton_expert_requested() and flags.triton_expert_available()
+        self.triton_cat_cast = flags.triton_cat_cast_requested()
+        self.batched_routers = flags.batched_routers_enabled() and num_groups > 1
+        if self.batched_routers:
+            check_batchable(list(self.private_routers))
+        self._declare_expert_banks(
+            [("stacked_public", self.public_experts), ("stacked_private", self._private_bank())]
+        )
+
+    # -- slots ---------------------------------------------------------------
+    def _private_bank(self) -> list[nn.Module]:
+        return [expert for column in self.private_experts for expert in column]
+
+    def _public_slots(self, public_output: RouterOutput, num_tokens: int) -> tuple[Tensor, Tensor]:
+        ids = public_output.topk_indices.reshape(num_tokens, self.public_top_k)
+        gates = public_output.gates.reshape(num_tokens, self.num_public_experts)
+        return ids, gates.gather(1, ids)
+
+    def _private_slots(self, private_outputs: list[RouterOutput], flat_group_gates: Tensor,
+                       num_tokens: int, selected: Tensor | None = None,
+                       stacked: tuple[Tensor, Tensor] | None = None) -> tuple[Tensor, Tensor, Tensor]:
+        """ids ``column * Q + expert`` and weights ``private_gate * column_gate`` for
+        the ``k_a * k_q`` private rows of every token, slot-major."""
+
+        k_a, k_q, q = self.num_groups_per_token, self.private_top_k, self.num_private_experts
+        if stacked is None:
+            gates = torch.stack([o.gates for o in private_outputs], dim=-2)
+            choices = torch.stack([o.topk_indices for o in private_outputs], dim=-2)
+        else:
+            gates, choices = stacked
+        gates = gates.reshape(num_tokens, self.num_groups, q)
+        choices = choices.reshape(num_tokens, self.num_groups, k_q)
+        if selected is None:
+            selected = torch.topk(flat_group_gates, k_a, dim=-1).indices
+        else:
+            selected = selected.reshape(num_tokens, k_a)
+        column_gate = flat_group_gates.gather(1, selected)
+        col = selected.unsqueeze(-1)
+        chosen = choices.gather(1, col.expand(-1, -1, k_q))
+        chosen_gates = gates.gather(1, col.expand(-1, -1, q)).gather(2, chosen)
+        ids = col * q + chosen
+        weights = chosen_gates * column_gate.unsqueeze(-1)
+        return ids.reshape(num_tokens, k_a * k_q), weights.reshape(num_tokens, k_a * k_q), selected
+
+    # -- routing -------------------------------------------------------------
+    def _route(self, x: Tensor, valid: Tensor, group_active: Tensor):
+        public_output = self.public_router(x, valid) if self.public_router is not None else None
+        if self.batched_routers:
+            outs, gates, choices = route_private_batched(
+                list(self.private_routers), x, valid, group_active, training=self.training
+            )
+            return public_output, outs, (gates, choices)
+        outs = [self.private_routers[g](x, valid & group_active[:, :, g])
+                for g in range(self.num_groups)]
+        return public_output, outs, None
+
+    # -- banks ---------------------------------------------------------------
+    def _bank(self, flat_x: Tensor, experts, stacked, ids: Tensor, weights: Tensor, group: int) -> Tensor:
+        return grouped_expert_combine(
+            flat_x, experts, ids, weights, group, fused_gate=self.fused_gate, stacked=stacked,
+            triton_index=self.triton_index, triton_fused=self.triton_fused,
+            triton_cat_cast=self.triton_cat_cast,
+        )
+
+    def _public_update(self, flat_x: Tensor, public_output: RouterOutput, num_tokens: int) -> Tensor:
+        ids, weights = self._public_slots(public_output, num_tokens)
+        return self._bank(flat_x, list(self.public_experts), self.stacked_public, ids, weights,
+                          self.public_top_k).reshape(num_tokens, -1)
+
+    def _private_per_slot(self, flat_x: Tensor, ids: Tensor, weights: Tensor) -> Tensor:
+        return self._bank(flat_x, self._private_bank(), self.stacked_private, ids, weights,
+                          self.private_top_k)
+
+    def _path_weights(self, x: Tensor) -> Tensor:
+        return F.softmax(self.path_gate(x).float(), dim=-1).to(x.dtype)
+
+    def _prologue(self, x: Tensor, valid: Tensor, group_gates: Tensor, group_active: Tensor):
+        flat_x = x.reshape(-1, self.dim)
+        num_tokens = flat_x.shape[0]
+        flat_gates = group_gates.reshape(num_tokens, self.num_groups)
+        public_output, private_outputs, stacked = self._route(x, valid, group_active)
+        public_update = (
+            self._public_update(flat_x, public_output, num_tokens).reshape_as(x)
+            if public_output is not None else None
+        )
+        return flat_x, num_tokens, flat_gates, public_output, private_outputs, stacked, public_update
+
+    # -- forwards ------------------------------------------------------------
+    def forward(self, x: Tensor, valid_token_mask: Tensor, group_gates: Tensor,
+                group_active_mask: Tensor, router_noise=None):
+        """Summed layout: ``(update [B,S,d], public_output, private_outputs)``."""
+
+        flat_x, n, flat_gates, pub_out, priv_outs, stacked, public_update = self._prologue(
+            x, valid_token_mask, group_gates, group_active_mask
+        )
+        ids, weights, _ = self._private_slots(priv_outs, flat_gates, n, stacked=stacked)
+        private_update = self._bank(
+            flat_x, self._private_bank(), self.stacked_private, ids, weights, ids.shape[1]
+        ).reshape_as(x)
+        if public_update is None:
+            return private_update.to(x.dtype), pub_out, priv_outs
+        alpha = self._path_weights(x)
+        update = alpha[..., 0:1] * public_update + alpha[..., 1:2] * private_update
+        return update.to(x.dtype), pub_out, priv_outs
+
+    def forward_per_slot(self, x: Tensor, valid_token_mask: Tensor, group_gates: Tensor,
+                         group_active_mask: Tensor, slot_groups: Tensor, router_noise=None):
+        """Slot layout: ``(public [B,S,d] | None, private [B,S,k_a,d], ...)``."""
+
+        flat_x, n, flat_gates, pub_out, priv_outs, stacked, public_update = self._prologue(
+            x, valid_token_mask, group_gates, group_active_mask
+        )
+        ids, weights, _ = self._private_slots(
+            priv_outs, flat_gates, n, selected=slot_groups.reshape(n, -1), stacked=stacked
+        )
+        per_slot = self._private_per_slot(flat_x, ids, weights).view(
+            x.shape[0], x.shape[1], -1, self.dim
+        )
+        return self._gate_split(x, public_update, per_slot, pub_out, priv_outs)
+
+    def forward_per_group(self, x: Tensor, valid_token_mask: Tensor, group_gates: Tensor,
+                          group_active_mask: Tensor, router_noise=None):
+        """Column layout: ``(public [B,S,d] | None, private [B,S,G,d], ...)``."""
+
+        flat_x, n, flat_gates, pub_out, priv_outs, stacked, public_update = self._prologue(
+            x, valid_token_mask, group_gates, group_active_mask
+        )
+        ids, weights, selected = self._private_slots(priv_outs, flat_gates, n, stacked=stacked)
+        per_slot = self._private_per_slot(flat_x, ids, weights)
+        index = selected.unsqueeze(-1).expand(-1, -1, self.dim)
+        per_group = flat_x.new_zeros(n, self.num_groups, self.dim).scatter_add(1, index, per_slot)
+        per_group = per_group.view(x.shape[0], x.shape[1], self.num_groups, self.dim)
+        return self._gate_split(x, public_update, per_group, pub_out, priv_outs)
+
+    def _gate_split(self, x, public_update, private_split, pub_out, priv_outs):
+        if public_update is None:
+            return None, private_split.to(x.dtype), pub_out, priv_outs
+        alpha = self._path_weights(x)
+        return (
+            (alpha[..., 0:1] * public_update).to(x.dtype),
+            (alpha[..., 1:2].unsqueeze(-1) * private_split).to(x.dtype),
+            pub_out,
+            priv_outs,
+        )

@@ -1,0 +1,194 @@
+"""Token-choice top-k routers of the expert pools.
+
+Mirrors ``RouterOutput`` / ``Router`` (nestor/backbones/nestor.py:320-593, the
+deterministic forward: score head, softmax, detached choice bias, top-k,
+``renorm`` / ``switch`` gate, scatter, validity mask) and the batched evaluation
+of a layer's ``G`` private routers (nestor/backbones/batched_router.py:97-240).
+Everything after the score GEMM -- softmax, biased top-k, gates -- is one HIP
+launch for the whole ``[tokens, (G,) choices]`` block.  Exploration noise and
+the bias update belong to the training loop and are not part of this path.
+
+``torch.topk`` leaves the order of equal scores open; this implementation (and
+its oracle) take equal biased scores lowest index first.
+"""
+
+from __future__ import annotations
+
+from typing import NamedTuple
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from nestor_amd import ops
+
+_ACTIVATIONS = {"gelu": F.gelu, "silu": F.silu, "relu": F.relu}
+
+
+class RouterOutput(NamedTuple):
+    scores: Tensor
+    softmax_probs: Tensor
+    gates: Tensor
+    topk_indices: Tensor
+    active_mask: Tensor
+    valid_token_mask: Tensor
+
+
+class ScoreMLP(nn.Module):
+    """Score head: ``Linear`` layers with an activation between them (none after
+    the last); ``hidden_dims=[]`` is the single linear map every registered arm uses."""
+
+    def __init__(self, input_dim: int, hidden_dims: list[int], output_dim: int,
+                 activation: str = "gelu", bias: bool = True) -> None:
+        super().__init__()
+        dims = [input_dim, *hidden_dims, output_dim]
+        self.layers = nn.ModuleList(
+            [nn.Linear(dims[i], dims[i + 1], bias=bias) for i in range(len(dims) - 1)]
+        )
+        self.activation = activation
+        self._activation_fn = _ACTIVATIONS[activation]
+        with torch.no_grad():
+            for layer in self.layers:
+                layer.weight.normal_(0.0, 1.0 / layer.in_features)
+                if layer.bias is not None:
+                    layer.bias.zero_()
+
+    def forward(self, x: Tensor) -> Tensor:
+        for layer in self.layers[:-1]:
+            x = self._activation_fn(layer(x))
+        return self.layers[-1](x)
+
+
+def _softmax_dtype(scores: Tensor) -> torch.dtype:
+    # F.softmax is on autocast's fp32 list; outside autocast it keeps the input dtype.
+    return torch.float32 if torch.is_autocast_enabled(scores.device.type) else scores.dtype
+
+
+def route_scores(
+    scores: Tensor, choice_bias: Tensor, top_k: int, gate_mode: str, mask: Tensor
+) -> tuple[Tensor, Tensor, Tensor]:
+    """``(softmax_probs, topk_indices, gates)`` for ``scores [..., C]``.
+
+    ``choice_bias`` is ``[C]`` or, for batched routers, ``[G, C]`` matching the
+    second-to-last axis of ``scores``; ``mask`` has the shape of ``scores[..., 0]``.
+    The top-k and, when no gradient is needed, the gates come from the HIP
+    kernel; with gradients the gates are rebuilt from differentiable torch ops on
+    the kernel's indices, in the reference's op order.
+    """
+
+    shape = scores.shape
+    c = shape[-1]
+    flat = scores.reshape(-1, c)
+    mode = 1 if gate_mode == "switch" else 0
+    probs, topk, gates = ops.router_topk(
+        flat.detach(), choice_bias.detach().float().reshape(-1, c), mask.reshape(-1), top_k, mode
+    )
+    topk = topk.view(*shape[:-1], top_k)
+    if torch.is_grad_enabled() and scores.requires_grad:
+        softmax_probs = F.softmax(scores, dim=-1)
+        if gate_mode == "switch":
+            topk_gates = F.softmax(scores.float(), dim=-1).gather(-1, topk).to(scores.dtype)
+        else:
+            topk_gates = F.softmax(scores.gather(-1, topk).float(), dim=-1).to(scores.dtype)
+        dense = torch.zeros_like(scores).scatter_add(-1, topk, topk_gates)
+        dense = dense * mask.unsqueeze(-1).to(dense.dtype)
+        return softmax_probs, topk, dense
+    return probs.view(shape).to(_softmax_dtype(scores)), topk, gates.view(shape)
+
+
+class Router(nn.Module):
+    """Top-k router over ``num_choices`` with a detached ``choice_bias`` buffer."""
+
+    def __init__(self, feature_dim: int, num_choices: int, num_choices_per_token: int,
+                 score_mlp_hidden_dims: list[int], score_mlp_activation: str = "gelu",
+                 noise_mlp_hidden_dims: list[int] | None = None,
+                 noise_mlp_activation: str = "gelu", *, loss_free_balancing: bool = False,
+                 bias_update_rate: float = 0.0, gate_mode: str = "renorm") -> None:
+        super().__init__()
+        if num_choices < 1:
+            raise ValueError("num_choices must be positive.")
+        if not 1 <= num_choices_per_token <= num_choices:
+            raise ValueError("num_choices_per_token must be in [1, num_choices].")
+        if gate_mode not in ("renorm", "switch"):
+            raise ValueError(f"gate_mode must be 'renorm' or 'switch', got {gate_mode!r}.")
+        self.feature_dim = feature_dim
+        self.num_choices = num_choices
+        self.num_choices_per_token = num_choices_per_token
+        self.loss_free_balancing = loss_free_balancing
+        self.bias_update_rate = bias_update_rate
+        self.gate_mode = gate_mode
+        self.score_mlp = ScoreMLP(feature_dim, score_mlp_hidden_dims, num_choices,
+                                  score_mlp_activation)
+        self.noise_mlp = None
+        self.register_buffer("choice_bias", torch.zeros(num_choices))
+
+    def forward(self, x: Tensor, valid_token_mask: Tensor, noise: Tensor | None = None) -> RouterOutput:
+        scores = self.score_mlp(x)
+        probs, topk, gates = route_scores(
+            scores, self.choice_bias, self.num_choices_per_token, self.gate_mode, valid_token_mask
+        )
+        return RouterOutput(scores, probs, gates, topk, gates > 0, valid_token_mask)
+
+
+def check_batchable(routers: list[Router]) -> None:
+    """Raise unless the routers can run as one batched router."""
+
+    if not routers:
+        raise ValueError("Need at least one router to batch.")
+
+    def signature(r: Router) -> tuple:
+        shape = tuple((l.in_features, l.out_features, l.bias is not None) for l in r.score_mlp.layers)
+        return (r.num_choices, r.num_choices_per_token, r.gate_mode, shape, r.score_mlp.activation)
+
+    if any(signature(r) != signature(routers[0]) for r in routers[1:]):
+        raise ValueError("Private routers differ in shape/gate mode; cannot batch them.")
+
+
+def batched_mlp(x: Tensor, mlps: list[ScoreMLP]) -> Tensor:
+    """``[N, G, d_out]``: ``G`` same-shaped heads on shared rows -- one GEMM for the
+    first layers (weights concatenated along the output axis), one ``[G]``-batched
+    matmul per later layer."""
+
+    heads = len(mlps)
+    w0 = torch.stack([m.layers[0].weight for m in mlps])
+    b0 = (
+        torch.stack([m.layers[0].bias for m in mlps]).reshape(-1)
+        if mlps[0].layers[0].bias is not None else None
+    )
+    hidden = F.linear(x, w0.reshape(heads * w0.shape[1], w0.shape[2]), b0)
+    hidden = hidden.view(x.shape[0], heads, w0.shape[1])
+    for index in range(1, len(mlps[0].layers)):
+        hidden = mlps[0]._activation_fn(hidden)
+        w = torch.stack([m.layers[index].weight for m in mlps])
+        hidden = torch.einsum("ngi,goi->ngo", hidden, w)
+        if mlps[0].layers[index].bias is not None:
+            hidden = hidden + torch.stack([m.layers[index].bias for m in mlps])
+    return hidden
+
+
+def route_private_batched(
+    routers: list[Router], x: Tensor, valid_token_mask: Tensor, group_active_mask: Tensor,
+    training: bool, noise: Tensor | None = None,
+) -> tuple[list[RouterOutput], Tensor, Tensor]:
+    """All ``G`` private routers of a layer in one pass: per-group outputs (views
+    of the stacked tensors, masked to ``valid & member``), stacked gates
+    ``[B, S, G, Q]`` and stacked choices ``[B, S, G, k]``."""
+
+    first = routers[0]
+    groups = len(routers)
+    batch, seq, dim = x.shape
+    scores = batched_mlp(x.reshape(batch * seq, dim), [r.score_mlp for r in routers]).view(
+        batch, seq, groups, first.num_choices
+    )
+    bias = torch.stack([r.choice_bias for r in routers])
+    member = valid_token_mask.unsqueeze(-1) & group_active_mask
+    probs, topk, gates = route_scores(
+        scores, bias, first.num_choices_per_token, first.gate_mode, member
+    )
+    active = gates > 0
+    outputs = [
+        RouterOutput(scores[:, :, g], probs[:, :, g], gates[:, :, g], topk[:, :, g],
+                     active[:, :, g], member[:, :, g])
+        for g in range(groups)
+    ]
+    return outputs, gates, topk

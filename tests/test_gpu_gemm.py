@@ -1,0 +1,122 @@
+"""Grouped GEMM kernels through the C ABI vs per-segment matmul (the
+reference's own CPU fallback, nestor/backbones/grouped_mm.py:97-104)."""
+
+import pytest
+import torch
+
+from oracle import bank as obank
+from oracle import plan as oplan
+from oracle import rows as orows
+from tests.helpers import gen, rel_l2, routing, zipf_ids
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(tokens, slots, banks, cuda, skew=False, capacity=0):
+    from nestor_amd.dispatch import dispatch_plan
+
+    ids = zipf_ids(1, tokens, slots, banks) if skew else routing(tokens, tokens, slots, banks)[0]
+    want = oplan.dispatch_plan(ids.reshape(-1), banks, slots, torch.bfloat16, capacity)
+    got = dispatch_plan(ids.reshape(-1).to(cuda), banks, slots, torch.bfloat16, capacity)
+    return want, got
+
+
+def _padded_input(want, cols, seed, scale=1.0):
+    a = (torch.randn(want.rows_pad, cols, generator=gen(seed)) * scale).to(torch.bfloat16)
+    return a * want.pad_valid.unsqueeze(1)  # slack rows are zero in every padded tensor
+
+
+SHAPES = [
+    # tokens, slots, banks, K, N, skew
+    (300, 2, 6, 40, 24, False),       # ragged everything (K, N multiples of 8 only)
+    (64, 1, 1, 64, 128, False),       # a single bank
+    (1000, 3, 20, 512, 1024, False),  # tiny config widths
+    (700, 2, 16, 200, 424, True),     # production-like odd widths, empty banks
+    (2048, 2, 8, 1024, 2048, False),
+]
+
+
+@pytest.mark.parametrize("tokens,slots,banks,K,N,skew", SHAPES)
+def test_segment_mm_forward_and_grads(cuda, tokens, slots, banks, K, N, skew):
+    from nestor_amd import segment_mm
+
+    want, got = _setup(tokens, slots, banks, cuda, skew)
+    a = _padded_input(want, K, 3)
+    b = (torch.randn(banks, K, N, generator=gen(4)) / K ** 0.5).to(torch.bfloat16)
+    ref = obank.segment_mm(a, b, want.offs)
+    ta = a.to(cuda).requires_grad_(True)
+    tb = b.to(cuda).requires_grad_(True)
+    out = segment_mm(ta, tb, got.offs)
+    assert out.shape == ref.shape and out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=2 ** -6, atol=1e-3)
+    assert rel_l2(out, ref) < 2e-3
+    go = _padded_input(want, N, 5)
+    out.backward(go.to(cuda))
+    # dA = go @ b^T per segment; dB[e] = a_seg^T @ go_seg (fp32 references)
+    bounds = [0] + want.offs.tolist()
+    da = torch.cat([go[bounds[i]:bounds[i + 1]].float() @ b[i].float().t() for i in range(banks)])
+    db = torch.stack([a[bounds[i]:bounds[i + 1]].float().t() @ go[bounds[i]:bounds[i + 1]].float()
+                      for i in range(banks)])
+    assert rel_l2(ta.grad, da) < 4e-3
+    assert rel_l2(tb.grad, db) < 4e-3
+    empty = want.counts == 0
+    if empty.any():
+        assert (tb.grad.cpu()[empty] == 0).all()  # every bank gets a gradient, zeros if unused
+
+
+@pytest.mark.parametrize("tokens,slots,banks,K,H,skew", [
+    (300, 2, 6, 40, 24, False), (1000, 3, 20, 512, 1024, False), (700, 2, 16, 200, 424, True),
+    (2048, 1, 4, 1024, 2048, False),
+])
+def test_upgate_swiglu_fused_matches_unfused(cuda, tokens, slots, banks, K, H, skew):
+    """The fused up|gate + SwiGLU kernel against the oracle chain with the
+    reference's rounding points, values and gradients."""
+
+    from nestor_amd import ops
+
+    want, got = _setup(tokens, slots, banks, cuda, skew)
+    x_pad = _padded_input(want, K, 6)
+    w_up = (torch.randn(banks, K, H, generator=gen(7)) / K ** 0.5).to(torch.bfloat16)
+    w_gate = (torch.randn(banks, K, H, generator=gen(8)) / K ** 0.5).to(torch.bfloat16)
+    ug_ref = obank.segment_mm(x_pad, torch.cat([w_up, w_gate], -1), want.offs)
+    hid_ref = orows.swiglu(ug_ref[:, :H], ug_ref[:, H:])
+    tx = x_pad.to(cuda).requires_grad_(True)
+    tu = w_up.to(cuda).requires_grad_(True)
+    tg = w_gate.to(cuda).requires_grad_(True)
+    up_gate, hidden = ops.upgate_swiglu_op(tx, tu, tg, got.tile_table, got.offs,
+                                           got.padded_starts, got.counts)
+    torch.testing.assert_close(up_gate.cpu().float(), ug_ref.float(), rtol=2 ** -6, atol=1e-3)
+    torch.testing.assert_close(hidden.cpu().float(), hid_ref.float(), rtol=2 ** -5, atol=2e-3)
+    assert rel_l2(hidden, hid_ref) < 3e-3
+    slack = want.pad_valid == 0
+    assert (hidden.cpu()[slack] == 0).all() and (up_gate.cpu()[slack] == 0).all()
+    gh = _padded_input(want, H, 9)
+    hidden.backward(gh.to(cuda))
+    # fp32 reference of the same chain from the bf16 operands
+    xf = x_pad.float().requires_grad_(True)
+    uf = w_up.float().requires_grad_(True)
+    gf = w_gate.float().requires_grad_(True)
+    bounds = [0] + want.offs.tolist()
+    outs = []
+    for i in range(banks):
+        seg = xf[bounds[i]:bounds[i + 1]]
+        outs.append(torch.nn.functional.silu(seg @ gf[i]) * (seg @ uf[i]))
+    torch.cat(outs).backward(gh.float())
+    assert rel_l2(tx.grad, xf.grad) < 1e-2
+    assert rel_l2(tu.grad, uf.grad) < 1e-2
+    assert rel_l2(tg.grad, gf.grad) < 1e-2
+
+
+def test_slack_tail_is_zero_filled(cuda):
+    """Rows behind the last segment belong to no bank: outputs there are zeros
+    even when the output buffer held garbage."""
+
+    from nestor_amd import ops
+
+    want, got = _setup(200, 1, 30, cuda)
+    a = _padded_input(want, 64, 1)
+    b = torch.randn(30, 64, 128, generator=gen(2)).to(torch.bfloat16)
+    out = ops.grouped_gemm_nn(a.to(cuda), b.to(cuda), got.tile_table)
+    tail = int((want.padded_starts + (want.counts + 15) // 16 * 16)[-1])
+    assert tail < want.rows_pad
+    assert (out.cpu()[tail:] == 0).all()

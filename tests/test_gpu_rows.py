@@ -1,0 +1,148 @@
+"""Row kernels through the C ABI vs the oracle: dispatch gather, SwiGLU,
+cat+cast and the weighted combine, forward and backward.  Tolerances are the
+reference's own for these kernels (tests/test_triton_expert_dispatch.py:55-58):
+copies and casts exact, bf16 math within two bf16 ulps."""
+
+import pytest
+import torch
+
+from oracle import plan as oplan
+from oracle import rows as orows
+from tests.helpers import gen, routing
+
+pytestmark = pytest.mark.gpu
+
+BF16_RTOL = 2.0 ** -6
+BF16_ATOL = 1e-3
+
+
+def _plan(ids, banks, cuda, capacity=0):
+    from nestor_amd.dispatch import dispatch_plan
+
+    slots = ids.shape[1]
+    want = oplan.dispatch_plan(ids.reshape(-1), banks, slots, torch.bfloat16, capacity)
+    got = dispatch_plan(ids.reshape(-1).to(cuda), banks, slots, torch.bfloat16, capacity)
+    return want, got
+
+
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tokens,slots,banks,dim", [(300, 3, 8, 40), (257, 6, 24, 200), (4096, 2, 16, 512)])
+def test_dispatch_rows_fwd_bwd(cuda, x_dtype, tokens, slots, banks, dim):
+    from nestor_amd import dispatch_rows
+
+    ids, _ = routing(tokens + slots, tokens, slots, banks)
+    want, got = _plan(ids, banks, cuda)
+    x = torch.randn(tokens, dim, generator=gen(1)).to(x_dtype)
+    ref = orows.dispatch_rows(x, want.pad_token, want.pad_valid, torch.bfloat16)
+    xg = x.to(cuda).requires_grad_(True)
+    out = dispatch_rows(xg, got.pad_token, got.pad_valid, got.row_dest, slots, torch.bfloat16)
+    assert out.dtype == torch.bfloat16
+    assert torch.equal(out.cpu(), ref)  # a gather and one rounding: exact
+    slack = want.pad_valid == 0
+    assert slack.any() and (out.cpu()[slack] == 0).all()
+    g = torch.randn(want.rows_pad, dim, generator=gen(2)).to(torch.bfloat16)
+    out.backward(g.to(cuda))
+    gref = orows.dispatch_rows_bwd(g, want.row_dest, tokens, slots, x_dtype)
+    assert xg.grad.dtype == x_dtype
+    # fp32 sums of <= 6 bf16 terms: only the summation order can differ
+    if x_dtype == torch.float32:
+        torch.testing.assert_close(xg.grad.cpu(), gref, rtol=1e-6, atol=1e-6)
+    else:
+        torch.testing.assert_close(xg.grad.cpu().float(), gref.float(), rtol=2.0 ** -7, atol=1e-6)
+
+
+@pytest.mark.parametrize("rows,hidden,fused", [(1000, 200, True), (37, 16, True), (1000, 200, False), (130, 4096, True)])
+def test_swiglu_fwd_bwd(cuda, rows, hidden, fused):
+    from nestor_amd import swiglu, swiglu_fused
+
+    g = gen(rows * 31 + hidden)
+    ug = (torch.randn(rows, 2 * hidden, generator=g) * 3).to(torch.bfloat16)
+    up, gate = ug[:, :hidden].contiguous(), ug[:, hidden:].contiguous()
+    ref = orows.swiglu(up, gate)
+    go = torch.randn(rows, hidden, generator=g).to(torch.bfloat16)
+    rup, rgate = orows.swiglu_bwd(go, up, gate)
+    if fused:
+        t = ug.to(cuda).requires_grad_(True)
+        out = swiglu_fused(t, hidden)
+        out.backward(go.to(cuda))
+        gup, ggate = t.grad[:, :hidden].cpu(), t.grad[:, hidden:].cpu()
+    else:
+        tu, tg = up.to(cuda).requires_grad_(True), gate.to(cuda).requires_grad_(True)
+        out = swiglu(tu, tg)
+        out.backward(go.to(cuda))
+        gup, ggate = tu.grad.cpu(), tg.grad.cpu()
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=BF16_RTOL, atol=BF16_ATOL)
+    torch.testing.assert_close(gup.float(), rup.float(), rtol=BF16_RTOL, atol=BF16_ATOL)
+    torch.testing.assert_close(ggate.float(), rgate.float(), rtol=BF16_RTOL, atol=BF16_ATOL)
+    # silu's exp may differ by an fp32 ulp before the bf16 rounding: rare 1-ulp flips only
+    assert (out.cpu() != ref).float().mean() < 0.01
+
+
+def test_cat_cast_bit_exact(cuda):
+    from nestor_amd import cat_cast
+
+    g = gen(5)
+    a = torch.randn(6, 40, 24, generator=g)
+    b = torch.randn(6, 40, 24, generator=g)
+    ref = orows.cat_cast(a, b, torch.bfloat16)
+    ta, tb = a.to(cuda).requires_grad_(True), b.to(cuda).requires_grad_(True)
+    out = cat_cast(ta, tb, torch.bfloat16)
+    assert out.shape == ref.shape and out.dtype == ref.dtype and out.is_contiguous()
+    assert torch.equal(out.cpu(), ref)
+    cot = torch.randn(ref.shape, generator=g).to(torch.bfloat16)
+    out.backward(cot.to(cuda))
+    assert torch.equal(ta.grad.cpu(), cot[..., :24].float())
+    assert torch.equal(tb.grad.cpu(), cot[..., 24:].float())
+    assert ta.grad.is_contiguous() and tb.grad.is_contiguous()
+
+
+@pytest.mark.parametrize("tokens,slots,group,banks,dim,out_dtype,w_dtype", [
+    (300, 2, 2, 8, 40, torch.float32, torch.float32),
+    (257, 6, 2, 24, 40, torch.float32, torch.float32),
+    (300, 4, 4, 8, 200, torch.bfloat16, torch.float32),
+    (512, 2, 1, 16, 512, torch.bfloat16, torch.bfloat16),
+    (512, 2, 1, 16, 512, torch.float32, torch.bfloat16),
+])
+def test_combine_rows_fwd_bwd(cuda, tokens, slots, group, banks, dim, out_dtype, w_dtype):
+    from nestor_amd import combine_rows
+
+    ids, weights = routing(tokens + slots, tokens, slots, banks)
+    weights = weights.to(w_dtype)
+    want, got = _plan(ids, banks, cuda)
+    y = (torch.randn(want.rows_pad, dim, generator=gen(7)) * 2).to(torch.bfloat16)
+    w = weights.reshape(-1)
+    ref = orows.combine_rows(y, want.row_dest, w, group, out_dtype)
+    eager = orows.combine_rows_eager(y, want.row_dest, w, group, out_dtype)
+    ty = y.to(cuda).requires_grad_(True)
+    tw = w.to(cuda).requires_grad_(True)
+    out = combine_rows(ty, got.row_dest, got.pad_src_row, got.pad_valid, tw, group, out_dtype)
+    assert out.dtype == out_dtype and out.shape == ref.shape
+    if out_dtype == torch.float32:
+        torch.testing.assert_close(out.cpu(), ref, rtol=1e-6, atol=1e-6)
+        torch.testing.assert_close(out.cpu(), eager, rtol=BF16_RTOL, atol=1e-2)
+    else:
+        torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=BF16_RTOL, atol=BF16_ATOL)
+        torch.testing.assert_close(out.cpu().float(), eager.float(), rtol=BF16_RTOL, atol=1e-2)
+    go = torch.randn(ref.shape, generator=gen(8)).to(out_dtype)
+    out.backward(go.to(cuda))
+    gy_ref, gw_ref = orows.combine_rows_bwd(go, y, want.pad_src_row, want.pad_valid, w, group)
+    torch.testing.assert_close(ty.grad.cpu().float(), gy_ref.float(), rtol=BF16_RTOL, atol=1e-6)
+    slack = want.pad_valid == 0
+    assert (ty.grad.cpu()[slack] == 0).all()
+    assert tw.grad.dtype == w_dtype
+    torch.testing.assert_close(tw.grad.cpu().float(), gw_ref.to(w_dtype).float(), rtol=1e-2 if w_dtype == torch.bfloat16 else 1e-4, atol=1e-2 if w_dtype == torch.bfloat16 else 1e-3)
+
+
+def test_identity_round_trip(cuda):
+    """combine(dispatch(x)) with unit weights sums each token's ``slots`` copies."""
+
+    from nestor_amd import combine_rows, dispatch_rows
+
+    tokens, slots, banks, dim = 500, 3, 12, 64
+    ids, _ = routing(9, tokens, slots, banks)
+    _, got = _plan(ids, banks, cuda)
+    x = torch.randint(-8, 8, (tokens, dim), generator=gen(4)).float()
+    xp = dispatch_rows(x.to(cuda), got.pad_token, got.pad_valid, got.row_dest, slots, torch.bfloat16)
+    ones = torch.ones(tokens * slots, device=cuda)
+    back = combine_rows(xp, got.row_dest, got.pad_src_row, got.pad_valid, ones, slots, torch.float32)
+    assert torch.equal(back.cpu(), slots * x)
