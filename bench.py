@@ -1,0 +1,300 @@
+"""Benchmark of the routed hybrid expert-MLP path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mlp_1b]
+
+A step is one forward + backward pass of the hot path over one batch of the
+1b-like workload (T = 32768 tokens, d = 2048, h = 4096, 16 public + 32 x 4
+private SwiGLU experts, top-2 columns -> top-1 private each, + top-1 public):
+column router, pool routers, index build, dispatch, grouped GEMMs with SwiGLU,
+weighted combine, and every gradient (inputs, routing weights, all three banks).
+Inputs are resident in HBM before the timed region.  One JSON line is printed.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
+
+
+def _event_ms(fn, iters: int) -> float:
+    """Average duration of ``fn`` over ``iters`` launches, from HIP events recorded
+    on the stream the kernels are launched on (torch's current stream)."""
+
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    fn()
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def kernel_breakdown(w, tensors, iters: int = 5) -> dict:
+    """Per-kernel timings of one private-bank call (the larger of the two), each
+    measured alone with HIP events, against the roofline that bounds it."""
+
+    from nestor_amd import ops
+    from nestor_amd.dispatch import dispatch_plan
+
+    dev = tensors.x.device
+    T, d, h = w.tokens, w.d_model, w.hidden
+    slots = w.k_columns * w.k_private
+    banks = w.columns * w.private
+    rows = T * slots
+    g = torch.Generator(device=dev).manual_seed(1)
+    ids = torch.randint(0, banks, (rows,), generator=g, device=dev)
+    weights = torch.rand(rows, generator=g, device=dev).to(torch.bfloat16)
+    w_up, w_gate, w_down = tensors.priv
+    out: dict = {}
+
+    def report(name, ms, flops=None, bytes_=None):
+        entry = {"ms": round(ms, 4)}
+        if flops is not None:
+            tf = flops / ms / 1e9
+            entry.update(tflops=round(tf, 1), frac_mfma_peak=round(tf / BF16_MFMA_PEAK_TFLOPS, 4))
+        if bytes_ is not None:
+            gbs = bytes_ / ms / 1e6
+            entry.update(gbs=round(gbs, 1), frac_hbm_peak=round(gbs / HBM_PEAK_GBS, 4))
+        out[name] = entry
+
+    plan = dispatch_plan(ids, banks, slots, torch.bfloat16)
+    rows_pad = plan.rows_pad
+    ms = _event_ms(lambda: dispatch_plan(ids, banks, slots, torch.bfloat16), iters)
+    report("index_build", ms, bytes_=rows * 8 + rows * 8 + 3 * rows_pad * 8 + rows_pad * 2 + banks * 20)
+
+    x = tensors.x
+    x_pad = ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid)
+    ms = _event_ms(lambda: ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid), iters)
+    report("dispatch_fwd", ms, bytes_=T * d * 2 + rows * d * 2 + rows * 8)
+
+    up_gate, hidden = ops.upgate_swiglu_fwd(x_pad, w_up, w_gate, plan.tile_table)
+    ms = _event_ms(lambda: ops.upgate_swiglu_fwd(x_pad, w_up, w_gate, plan.tile_table), iters)
+    report("gemm_upgate_swiglu", ms, flops=2.0 * rows * d * 2 * h)
+    out["gemm_upgate_swiglu"]["flops_per_launch"] = 2.0 * rows * d * 2 * h
+
+    y_pad = ops.grouped_gemm_nn(hidden, w_down, plan.tile_table)
+    ms = _event_ms(lambda: ops.grouped_gemm_nn(hidden, w_down, plan.tile_table), iters)
+    report("gemm_down", ms, flops=2.0 * rows * h * d)
+
+    o = ops.combine_rows_fwd(y_pad, plan.row_dest, weights, slots, torch.bfloat16, True)
+    ms = _event_ms(lambda: ops.combine_rows_fwd(y_pad, plan.row_dest, weights, slots, torch.bfloat16, True), iters)
+    report("combine_fwd", ms, bytes_=rows * d * 2 + rows * (8 + 2) + (rows // slots) * d * 2)
+
+    go = tensors.grad_out
+    ms = _event_ms(lambda: ops.combine_rows_bwd(go, y_pad, plan.pad_src_row, plan.pad_valid, weights, slots, True), iters)
+    report("combine_bwd", ms, bytes_=(rows // slots) * d * 2 + rows * d * 2 + rows * d * 2 + rows * 4)
+    gy, _ = ops.combine_rows_bwd(go, y_pad, plan.pad_src_row, plan.pad_valid, weights, slots, True)
+
+    ms = _event_ms(lambda: ops.grouped_gemm_nt(gy, w_down, plan.tile_table), iters)
+    report("gemm_dgrad_down", ms, flops=2.0 * rows * h * d)
+    gh = ops.grouped_gemm_nt(gy, w_down, plan.tile_table)
+
+    ms = _event_ms(lambda: ops.grouped_gemm_tn(hidden, gy, plan.offs, plan.padded_starts, plan.counts), iters)
+    report("gemm_wgrad_down", ms, flops=2.0 * rows * h * d)
+
+    ms = _event_ms(lambda: ops.swiglu_bwd(gh, up_gate, h), iters)
+    report("swiglu_bwd", ms, bytes_=rows * h * 2 * (1 + 2 + 2))
+    gug = ops.swiglu_bwd(gh, up_gate, h)
+
+    ms = _event_ms(lambda: ops.grouped_gemm_nt_upgate(gug, w_up, w_gate, plan.tile_table), iters)
+    report("gemm_dgrad_upgate", ms, flops=2.0 * rows * d * 2 * h)
+    gx_pad = ops.grouped_gemm_nt_upgate(gug, w_up, w_gate, plan.tile_table)
+
+    ms = _event_ms(lambda: ops.grouped_gemm_tn(x_pad, gug[:, :h], plan.offs, plan.padded_starts, plan.counts), iters)
+    report("gemm_wgrad_up(one of 2)", ms, flops=2.0 * rows * d * h)
+
+    ms = _event_ms(lambda: ops.dispatch_rows_bwd(gx_pad, plan.row_dest, T, slots, torch.bfloat16), iters)
+    report("dispatch_bwd", ms, bytes_=rows * d * 2 + T * d * 2)
+    del o
+    return out
+
+
+def _log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def cpu_baseline(w, seed: int, target_seconds: float = 15.0) -> dict:
+    """The reference's CPU eager path (per-expert sparse loop under bf16 autocast,
+    forward + backward) on a bounded slice of the same workload: 1/16 of the
+    tokens over 1/16 of the banks, so every expert sees as many rows as in the
+    full workload and the work per token is unchanged."""
+
+    from oracle import bank as obank
+    from oracle import router as orouter
+
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    shrink = 16
+    columns = max(w.k_columns, w.columns // shrink)
+    public = max(w.k_public, w.public // shrink)
+    sample = max(64, w.tokens * columns // w.columns)
+    d, h = w.d_model, w.hidden
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(sample, d, generator=g).bfloat16().float().requires_grad_(True)
+    go = torch.randn(sample, d, generator=g)
+    ones = torch.ones(sample, dtype=torch.bool)
+    col = orouter.route(torch.randn(sample, columns, generator=g), torch.zeros(columns),
+                        w.k_columns, "renorm", ones)
+    pub = orouter.route(torch.randn(sample, public, generator=g), torch.zeros(public),
+                        w.k_public, "renorm", ones)
+    priv = orouter.route(torch.randn(sample, columns, w.private, generator=g),
+                         torch.zeros(columns, w.private), w.k_private, "switch",
+                         torch.ones(sample, columns, dtype=torch.bool))
+    ids, wts, _ = orouter.private_slots(priv.gates, priv.topk_indices, col.gates, w.k_columns)
+    pub_ids, pub_w = orouter.public_slots(pub.gates, pub.topk_indices)
+    banks = []
+    for n in (public, columns * w.private):
+        banks.append(tuple(
+            (torch.randn(n, a, b, generator=g) * w.weight_std).requires_grad_(True)
+            for a, b in ((d, h), (d, h), (h, d))
+        ))
+
+    def step():
+        for bank in banks:
+            for t in bank:
+                t.grad = None
+        x.grad = None
+        out = torch.zeros(sample, d)
+        with torch.autocast("cpu", dtype=torch.bfloat16):
+            obank.accumulate_sparse_expert_bank(
+                out, x, *banks[0], obank.dense_weights(pub_ids, pub_w, public))
+            obank.accumulate_sparse_expert_bank(
+                out, x, *banks[1], obank.dense_weights(ids, wts, columns * w.private))
+        out.backward(go)
+
+    _log(f"cpu baseline: {sample} tokens, {public}+{columns}x{w.private} experts, {cores} threads")
+    step()  # warm-up
+    times = []
+    t_end = time.perf_counter() + target_seconds
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 10):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+        _log(f"cpu baseline pass {len(times)}: {times[-1]:.2f} s")
+    med = statistics.median(times)
+    return {
+        "value": round(sample / med, 1),
+        "unit": "tokens/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{sample} of {w.tokens} tokens over {public}+{columns}x{w.private} of "
+                  f"{w.public}+{w.columns}x{w.private} experts (same rows per expert as the full "
+                  f"workload), fwd+bwd, per-expert sparse loop under cpu bf16 autocast, "
+                  f"median of {len(times)} passes",
+    }
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="mlp_1b")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-breakdown", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU's share of the expert MLP: run it with --gpus 1 "
+                 "(the path shards by tokens; there is no multi-GPU leg in this build)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the HIP kernels have no CPU fallback)")
+
+    from nestor_amd import _lib
+    from nestor_amd.workloads import WORKLOADS, build_pool, expert_mlp_step, make_tensors
+
+    _lib.load()
+    _log("library loaded; building workload")
+    w = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    tensors = make_tensors(w, args.seed, dev)
+    column_router, pool = build_pool(w, tensors)
+    params = list(column_router.parameters()) + list(pool.parameters())
+    x = tensors.x.clone().requires_grad_(True)
+    grad_out = tensors.grad_out if w.backward else None
+
+    def step():
+        for p in params:
+            p.grad = None
+        x.grad = None
+        expert_mlp_step(w, column_router, pool, x, grad_out)
+
+    _log("workload resident; warm-up")
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _log("timing")
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    tokens_per_s = w.tokens * args.steps / elapsed
+    flops = w.gemm_flops()
+    step_tflops = flops / (ms_per_step * 1e-3) / 1e12
+
+    _log(f"{ms_per_step:.3f} ms/step; per-kernel breakdown")
+    for p in params:
+        p.grad = None
+    x.grad = None
+    breakdown = {} if args.no_breakdown else kernel_breakdown(w, tensors)
+    dom = breakdown.get("gemm_upgate_swiglu")
+    roofline = None
+    if dom:
+        roofline = {
+            "bound": "mfma",
+            "kernel": "grouped_gemm_kernel<kNNUpGate> (private bank up|gate + SwiGLU)",
+            "achieved": dom["tflops"],
+            "peak": BF16_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": dom["frac_mfma_peak"],
+            "traffic": None,
+        }
+    result = {
+        "metric": "expert-MLP fwd+bwd tokens/s @1b shape, 1 GPU; % bf16 MFMA / HBM peak",
+        "value": round(tokens_per_s, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name}: T={w.tokens} d={w.d_model} h={w.hidden} experts={w.public}+"
+                        f"{w.columns}x{w.private}, top-{w.k_columns} columns -> top-{w.k_private} "
+                        f"private + top-{w.k_public} public, fwd{'+bwd' if w.backward else ''}",
+            "seed": args.seed,
+        },
+        "expert_gemm_tflops": round(step_tflops, 1),
+        "expert_gemm_frac_mfma_peak": round(step_tflops / BF16_MFMA_PEAK_TFLOPS, 4),
+        "gemm_flops_per_step": flops,
+        "roofline": roofline,
+        "kernels": breakdown,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(w, args.seed)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -93,6 +93,35 @@ class StackedExpertBank(nn.Module):
         self.b_down = owner([e.layers[1].bias for e in experts]) if biased else None
         self.install_views(experts)
 
+    @classmethod
+    def from_tensors(cls, w_up: Tensor, w_gate: Tensor | None, w_down: Tensor) -> "StackedExpertBank":
+        """A bias-free bank that adopts already-stacked tensors (``[E, d_in, h]``,
+        ``[E, d_in, h]`` or None, ``[E, h, d_out]``) as its owners without going
+        through per-expert modules -- how a checkpoint in the stacked layout or a
+        synthetic benchmark bank enters."""
+
+        bank = cls.__new__(cls)
+        nn.Module.__init__(bank)
+        bank.num_experts = w_up.shape[0]
+        bank.gated = w_gate is not None
+        bank.w_up = nn.Parameter(w_up)
+        bank.w_gate = nn.Parameter(w_gate) if w_gate is not None else None
+        bank.w_down = nn.Parameter(w_down)
+        bank.b_up = None
+        bank.b_down = None
+        return bank
+
+    def expert_views(self, activation: str = "silu") -> list["ExpertView"]:
+        """Per-expert read-only handles with the attribute surface the grouped
+        path inspects (``gated``, ``activation``, ``layers[i].weight/.bias``,
+        ``gate.weight``), as views of the owners."""
+
+        cached = self.__dict__.get("_views")
+        if cached is None or cached[0] != activation:
+            views = [ExpertView(self, i, activation) for i in range(self.num_experts)]
+            self.__dict__["_views"] = cached = (activation, views)
+        return cached[1]
+
     def install_views(self, experts: Sequence[nn.Module]) -> None:
         """Re-point every expert's ``weight`` / ``bias`` at a view of the owners;
         the per-expert entries leave ``_parameters`` so the model exposes each
@@ -119,6 +148,39 @@ class StackedExpertBank(nn.Module):
             self.w_gate.to(dtype) if self.w_gate is not None else None,
             self.w_down.to(dtype),
         )
+
+
+class _LinearView:
+    def __init__(self, weight: Tensor, bias: Tensor | None) -> None:
+        self.weight = weight
+        self.bias = bias
+
+
+class ExpertView:
+    """Expert ``index`` of a stacked bank, duck-typed like ``SwigluExpert``.  The
+    weight views are formed on access, so they always reflect the bank's current
+    tensors (after ``.to()`` / ``.cuda()`` too) and a list of views costs nothing
+    until one is read."""
+
+    def __init__(self, bank: StackedExpertBank, index: int, activation: str) -> None:
+        self._bank = bank
+        self._index = index
+        self.gated = bank.gated
+        self.activation = activation
+        self._activation_fn = _ACTIVATIONS[activation]
+
+    @property
+    def layers(self) -> list[_LinearView]:
+        b, i = self._bank, self._index
+        return [
+            _LinearView(b.w_up[i].t(), b.b_up[i] if b.b_up is not None else None),
+            _LinearView(b.w_down[i].t(), b.b_down[i] if b.b_down is not None else None),
+        ]
+
+    @property
+    def gate(self) -> _LinearView | None:
+        b = self._bank
+        return _LinearView(b.w_gate[self._index].t(), None) if b.gated else None
 
 
 class StackedBanksMixin:

@@ -38,6 +38,7 @@ class DispatchPlan(NamedTuple):
     row_kept: Tensor
     tile_table: Tensor
     capacity: int
+    kept_counts: Tensor  # rows of each bank that own a padded slot (== counts when dropless)
 
 
 def dispatch_plan(
@@ -64,7 +65,7 @@ def dispatch_plan(
     return DispatchPlan(
         rows, ops.rows_pad_for(rows, num_banks), offs, row_dest, pad_token, pad_src_row,
         eid_pad, pad_valid, order, counts, raw_starts, padded_starts, row_kept, tile_table,
-        capacity,
+        capacity, counts.clamp(max=capacity) if capacity > 0 else counts,
     )
 
 

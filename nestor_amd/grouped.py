@@ -77,7 +77,7 @@ def _plan_mm(a: Tensor, b: Tensor, plan: DispatchPlan) -> Tensor:
     """``segment_mm`` driven by a plan: its tile table skips the slack tail and
     the weight gradient contracts over real rows only."""
 
-    return ops.grouped_mm_op(a, b, plan.tile_table, plan.offs, plan.padded_starts, plan.counts)
+    return ops.grouped_mm_op(a, b, plan.tile_table, plan.offs, plan.padded_starts, plan.kept_counts)
 
 
 def _bank_weights(
@@ -120,7 +120,7 @@ def _expert_rows_padded(
     if hip_fused and gated and not biased:
         # Both stacked banks read in place; SwiGLU in the GEMM epilogue.
         _up_gate, hidden = ops.upgate_swiglu_op(
-            x_pad, w_up, w_gate, plan.tile_table, plan.offs, plan.padded_starts, plan.counts
+            x_pad, w_up, w_gate, plan.tile_table, plan.offs, plan.padded_starts, plan.kept_counts
         )
         return _plan_mm(hidden, w_down, plan)
 

@@ -121,9 +121,62 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
             [("stacked_public", self.public_experts), ("stacked_private", self._private_bank())]
         )
 
+    @classmethod
+    def from_stacked(cls, dim: int, num_groups: int, num_groups_per_token: int,
+                     stacked_public, stacked_private, public_top_k: int, private_top_k: int,
+                     *, private_gate_mode: str = "switch",
+                     router_score_mlp_hidden_dims: list[int] | None = None) -> "ExpertPoolMLP":
+        """A pool around banks that already exist in the stacked layout
+        (``StackedExpertBank``; private bank index ``column * Q + expert``).  No
+        per-expert modules are built: the banks are the only owners of the expert
+        weights, which is how a stacked-layout checkpoint or a large synthetic
+        bank enters without materialising ``P + G*Q`` separate modules first."""
+
+        self = cls.__new__(cls)
+        nn.Module.__init__(self)
+        p = stacked_public.num_experts if stacked_public is not None else 0
+        q = stacked_private.num_experts // num_groups
+        self.dim, self.num_groups, self.num_groups_per_token = dim, num_groups, num_groups_per_token
+        self.num_public_experts, self.public_top_k = p, public_top_k
+        self.num_private_experts, self.private_top_k = q, private_top_k
+        self.private_gate_mode = private_gate_mode
+        self.has_public_pool = p > 0
+        self.public_hidden_dim = stacked_public.w_up.shape[-1] if p > 0 else 0
+        self.private_hidden_dim = stacked_private.w_up.shape[-1]
+        hidden = router_score_mlp_hidden_dims or []
+        self.public_router = Router(dim, p, public_top_k, hidden) if p > 0 else None
+        self.private_routers = nn.ModuleList(
+            [Router(dim, q, private_top_k, hidden, gate_mode=private_gate_mode)
+             for _ in range(num_groups)]
+        )
+        self.public_experts = None
+        self.private_experts = None
+        if p > 0:
+            self.path_gate = Linear2(dim, 2, bias=False)
+            with torch.no_grad():
+                self.path_gate.weight.zero_()
+        else:
+            self.path_gate = None
+        self.grouped_dispatch = None
+        self.fused_gate = True
+        self.triton_index = self.triton_fused = True
+        self.triton_cat_cast = True
+        self.batched_routers = num_groups > 1
+        self._stacked_bank_specs, self._stacked_view_sources = [], []
+        self.stacked_public = stacked_public
+        self.stacked_private = stacked_private
+        return self
+
     # -- slots ---------------------------------------------------------------
     def _private_bank(self) -> list[nn.Module]:
+        if self.private_experts is None:
+            return self.stacked_private.expert_views()
         return [expert for column in self.private_experts for expert in column]
+
+    def _public_bank(self) -> list[nn.Module]:
+        if self.public_experts is None:
+            return self.stacked_public.expert_views()
+        return list(self.public_experts)
 
     def _public_slots(self, public_output: RouterOutput, num_tokens: int) -> tuple[Tensor, Tensor]:
         ids = public_output.topk_indices.reshape(num_tokens, self.public_top_k)
@@ -178,7 +231,7 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
 
     def _public_update(self, flat_x: Tensor, public_output: RouterOutput, num_tokens: int) -> Tensor:
         ids, weights = self._public_slots(public_output, num_tokens)
-        return self._bank(flat_x, list(self.public_experts), self.stacked_public, ids, weights,
+        return self._bank(flat_x, self._public_bank(), self.stacked_public, ids, weights,
                           self.public_top_k).reshape(num_tokens, -1)
 
     def _private_per_slot(self, flat_x: Tensor, ids: Tensor, weights: Tensor) -> Tensor:

@@ -1,0 +1,144 @@
+"""Synthetic workloads of the expert-MLP measurement configs.
+
+Every config routes each token to its top-2 of ``G`` columns, to the top-1 of
+``Q`` private experts inside each chosen column, and to the top-1 of ``P`` public
+experts: three weighted assignments per token, issued as one public bank call
+(``slots = 1``) and one private bank call (``slots = 2``).  Activations are
+``N(0, 1)`` rounded to bf16, router heads ``N(0, 0.02)``, expert banks
+``N(0, std)`` in the stacked layout ``w_up / w_gate [E, d, h]``,
+``w_down [E, h, d]`` with the private bank indexed ``column * Q + expert``.
+Draws use a seeded generator on the device the tensors live on; copy them to the
+other side to compare implementations on identical bits.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+from torch import Tensor
+
+
+@dataclass(frozen=True)
+class Workload:
+    name: str
+    tokens: int
+    d_model: int
+    hidden: int
+    public: int      # P
+    columns: int     # G
+    private: int     # Q per column
+    weight_std: float
+    router_std: float = 0.02
+    k_columns: int = 2
+    k_private: int = 1
+    k_public: int = 1
+    backward: bool = True
+
+    @property
+    def experts(self) -> int:
+        return self.public + self.columns * self.private
+
+    @property
+    def assignments(self) -> int:
+        return self.k_public + self.k_columns * self.k_private
+
+    def gemm_flops(self, backward: bool | None = None) -> float:
+        """``2 * rows * K * N`` per GEMM over real rows: forward ``18 T d h`` at three
+        assignments per token, backward twice that."""
+
+        fwd = 6.0 * self.assignments * self.tokens * self.d_model * self.hidden
+        bwd = self.backward if backward is None else backward
+        return fwd * (3.0 if bwd else 1.0)
+
+
+WORKLOADS = {
+    "tiny_100m": Workload("tiny_100m", 4096, 512, 1024, 4, 8, 2, 0.02, backward=False),
+    "mlp_200m": Workload("mlp_200m", 16384, 1024, 2048, 8, 16, 4, 0.02),
+    "mlp_1b": Workload("mlp_1b", 32768, 2048, 4096, 16, 32, 4, 0.014),
+}
+
+
+@dataclass
+class WorkloadTensors:
+    x: Tensor            # [T, d] bf16
+    grad_out: Tensor     # [T, d] bf16
+    w_columns: Tensor    # [G, d]
+    w_public: Tensor     # [P, d]
+    w_private: Tensor    # [G, Q, d]
+    pub: tuple[Tensor, Tensor, Tensor]   # w_up, w_gate, w_down of the public bank
+    priv: tuple[Tensor, Tensor, Tensor]  # ... of the flattened private bank
+
+
+def make_tensors(w: Workload, seed: int, device: torch.device | str,
+                 weight_dtype: torch.dtype = torch.bfloat16) -> WorkloadTensors:
+    device = torch.device(device)
+    g = torch.Generator(device=device).manual_seed(seed)
+
+    def randn(*shape: int, std: float = 1.0, dtype: torch.dtype = torch.float32) -> Tensor:
+        # Drawn bank by bank so the fp32 staging buffer stays small at the 1b shape.
+        if len(shape) == 3 and shape[0] * shape[1] * shape[2] > (1 << 26):
+            out = torch.empty(shape, dtype=dtype, device=device)
+            for i in range(shape[0]):
+                out[i] = (torch.randn(shape[1:], generator=g, device=device) * std).to(dtype)
+            return out
+        return (torch.randn(shape, generator=g, device=device) * std).to(dtype)
+
+    def bank(n: int) -> tuple[Tensor, Tensor, Tensor]:
+        return (
+            randn(n, w.d_model, w.hidden, std=w.weight_std, dtype=weight_dtype),
+            randn(n, w.d_model, w.hidden, std=w.weight_std, dtype=weight_dtype),
+            randn(n, w.hidden, w.d_model, std=w.weight_std, dtype=weight_dtype),
+        )
+
+    x = randn(w.tokens, w.d_model, dtype=torch.bfloat16)
+    grad_out = randn(w.tokens, w.d_model, dtype=torch.bfloat16)
+    w_columns = randn(w.columns, w.d_model, std=w.router_std)
+    w_public = randn(w.public, w.d_model, std=w.router_std)
+    w_private = randn(w.columns, w.private, w.d_model, std=w.router_std)
+    return WorkloadTensors(x, grad_out, w_columns, w_public, w_private,
+                           bank(w.public), bank(w.columns * w.private))
+
+
+def build_pool(w: Workload, t: WorkloadTensors):
+    """(column_router, pool) on the tensors' device, sharing storage with ``t``."""
+
+    from nestor_amd.bank import StackedExpertBank
+    from nestor_amd.pool import ExpertPoolMLP
+    from nestor_amd.router import Router
+
+    dtype = t.pub[0].dtype
+    pool = ExpertPoolMLP.from_stacked(
+        w.d_model, w.columns, w.k_columns,
+        StackedExpertBank.from_tensors(*t.pub), StackedExpertBank.from_tensors(*t.priv),
+        w.k_public, w.k_private, private_gate_mode="switch",
+    )
+    column_router = Router(w.d_model, w.columns, w.k_columns, [])
+    with torch.no_grad():
+        def install(router, weight):
+            lin = router.score_mlp.layers[0]
+            lin.weight = torch.nn.Parameter(weight.to(dtype))
+            lin.bias = None
+        install(column_router, t.w_columns)
+        install(pool.public_router, t.w_public)
+        for g, r in enumerate(pool.private_routers):
+            install(r, t.w_private[g])
+        # a non-degenerate path gate (the zero init is an exact 0.5 / 0.5 split)
+        pool.path_gate.weight = torch.nn.Parameter(
+            (0.02 * torch.ones_like(pool.path_gate.weight)).to(dtype)
+        )
+    return column_router.to(t.x.device), pool.to(t.x.device)
+
+
+def expert_mlp_step(w: Workload, column_router, pool, x: Tensor, grad_out: Tensor | None):
+    """One pass of the hot path over one batch: column router -> pool routers ->
+    public + private bank calls -> weighted combine (+ backward when ``grad_out``
+    is given).  Returns the ``[T, d]`` update."""
+
+    x3 = x.view(1, w.tokens, w.d_model)
+    valid = torch.ones(1, w.tokens, dtype=torch.bool, device=x.device)
+    col = column_router(x3, valid)
+    update, _pub, _priv = pool(x3, valid, col.gates, col.active_mask)
+    if grad_out is not None:
+        update.backward(grad_out.view_as(update))
+    return update

@@ -1,0 +1,185 @@
+"""Whole bank calls (plan -> dispatch -> grouped GEMMs + SwiGLU -> combine) and the
+pool on the HIP path vs the oracle: the unrounded fp32 gold (rel-L2 <= 1e-2 for
+outputs and every gradient) and the oracle chain with the reference's rounding
+points (the reference's own bank tolerance, rtol 2^-6 / atol 1e-2,
+tests/test_triton_expert_dispatch.py:307)."""
+
+import pytest
+import torch
+
+from oracle import bank as obank
+from oracle import plan as oplan
+from tests.helpers import bank_weights, gen, rel_l2, routing, zipf_ids
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2  # rel-L2 vs fp32 for bf16 outputs and gradients
+
+
+def _hip_bank(cuda, x, w3, ids, weights, group, *, fused, capacity=0, autocast=False):
+    from nestor_amd import StackedExpertBank, grouped_expert_combine
+
+    bank = StackedExpertBank.from_tensors(*[t.clone() for t in w3]).to(cuda)
+    tx = x.detach().clone().to(cuda).requires_grad_(True)
+    tw = weights.detach().clone().to(cuda).requires_grad_(True)
+
+    def call():
+        return grouped_expert_combine(
+            tx, bank.expert_views(), ids.to(cuda), tw, group, fused_gate=True, stacked=bank,
+            triton_index=True, triton_fused=fused, capacity=capacity,
+        )
+
+    if autocast:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = call()
+    else:
+        out = call()
+    return bank, tx, tw, out
+
+
+def _gold(x, w3, ids, weights, group, go, row_kept=None, device="cpu"):
+    xs = x.detach().float().to(device).clone().requires_grad_(True)
+    ws = weights.detach().float().to(device).clone().requires_grad_(True)
+    w3f = [t.detach().float().to(device).clone().requires_grad_(True) for t in w3]
+    rk = None if row_kept is None else row_kept.to(device)
+    out = obank.gold_combine(xs, *w3f, ids.to(device), ws, group, rk)
+    out.backward(go.float().to(device))
+    return out.detach(), xs.grad, ws.grad, [t.grad for t in w3f]
+
+
+CASES = [
+    # name, tokens, d, h, banks, slots, group, std
+    ("tiny public", 4096, 512, 1024, 4, 1, 1, 0.02),
+    ("tiny private per-slot", 4096, 512, 1024, 16, 2, 1, 0.02),
+    ("tiny private summed", 4096, 512, 1024, 16, 2, 2, 0.02),
+    ("odd widths", 1000, 200, 424, 24, 6, 2, 0.05),
+]
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("name,tokens,d,h,banks,slots,group,std", CASES)
+def test_bank_fwd_bwd_vs_gold(cuda, name, tokens, d, h, banks, slots, group, std, fused):
+    ids, weights = routing(tokens, tokens, slots, banks)
+    weights = weights.bfloat16()
+    x = torch.randn(tokens, d, generator=gen(0)).bfloat16()
+    w3 = bank_weights(1, banks, d, h, std, torch.bfloat16)
+    go = torch.randn(tokens, slots // group, d, generator=gen(2)).bfloat16()
+    bank, tx, tw, out = _hip_bank(cuda, x, w3, ids, weights, group, fused=fused)
+    assert out.shape == (tokens, slots // group, d) and out.dtype == torch.bfloat16
+    out.backward(go.to(cuda))
+    ref, gx, gw, gw3 = _gold(x, w3, ids, weights, group, go)
+    assert rel_l2(out, ref) < TOL, name
+    assert rel_l2(tx.grad, gx) < TOL
+    assert rel_l2(tw.grad, gw) < TOL
+    for got, want, n in zip((bank.w_up.grad, bank.w_gate.grad, bank.w_down.grad), gw3,
+                            ("w_up", "w_gate", "w_down")):
+        assert got.dtype == torch.bfloat16
+        assert rel_l2(got, want) < TOL, n
+    # the oracle chain with the reference's rounding points
+    emu = obank.grouped_expert_combine(x, *w3, ids, weights, group, torch.bfloat16)
+    torch.testing.assert_close(out.cpu().float(), emu.float(), rtol=2 ** -6, atol=1e-2)
+
+
+def test_bank_fp32_stream_under_autocast(cuda):
+    """The production dtype flow: fp32 residual stream and fp32 owners under bf16
+    autocast; output and x / weight gradients come back in fp32."""
+
+    tokens, d, h, banks, slots, group = 600, 64, 96, 6, 2, 2
+    ids, weights = routing(5, tokens, slots, banks)
+    x = torch.randn(tokens, d, generator=gen(3))
+    w3 = bank_weights(4, banks, d, h, 0.1, torch.float32)
+    go = torch.randn(tokens, 1, d, generator=gen(5))
+    for fused in (True, False):
+        bank, tx, tw, out = _hip_bank(cuda, x, w3, ids, weights, group, fused=fused, autocast=True)
+        assert out.dtype == torch.float32
+        out.backward(go.to(cuda))
+        ref, gx, gw, gw3 = _gold(x, w3, ids, weights, group, go)
+        assert rel_l2(out, ref) < TOL
+        assert tx.grad.dtype == torch.float32 and rel_l2(tx.grad, gx) < TOL
+        assert tw.grad.dtype == torch.float32 and rel_l2(tw.grad, gw) < TOL
+        for got, want in zip((bank.w_up.grad, bank.w_gate.grad, bank.w_down.grad), gw3):
+            assert got.dtype == torch.float32 and rel_l2(got, want) < TOL
+        emu = obank.grouped_expert_combine(x, *w3, ids, weights, group, torch.bfloat16)
+        torch.testing.assert_close(out.cpu(), emu, rtol=2 ** -6, atol=1e-2)
+
+
+def test_skewed_bank_with_capacity_drop(cuda):
+    """Zipf-skewed routing with empty banks; capacity factor 1.25 drops the
+    overflow in stable token order and dropped rows contribute exactly zero."""
+
+    tokens, d, h, banks, slots, group = 4096, 256, 512, 64, 2, 2
+    ids = zipf_ids(0, tokens, slots, banks)
+    weights = torch.rand(tokens, slots, generator=gen(1)).bfloat16()
+    x = torch.randn(tokens, d, generator=gen(2)).bfloat16()
+    w3 = bank_weights(3, banks, d, h, 0.05, torch.bfloat16)
+    go = torch.randn(tokens, 1, d, generator=gen(4)).bfloat16()
+    cap = oplan.capacity_for(tokens * slots, banks, 1.25)
+    plan = oplan.dispatch_plan(ids.reshape(-1), banks, slots, torch.bfloat16, cap)
+    assert (plan.row_kept == 0).any() and (plan.counts == 0).any()
+    for capacity, kept in ((0, None), (cap, plan.row_kept)):
+        bank, tx, tw, out = _hip_bank(cuda, x, w3, ids, weights, group, fused=True, capacity=capacity)
+        out.backward(go.to(cuda))
+        ref, gx, gw, gw3 = _gold(x, w3, ids, weights, group, go, kept)
+        assert rel_l2(out, ref) < TOL
+        assert rel_l2(tx.grad, gx) < TOL
+        assert rel_l2(tw.grad, gw) < TOL
+        for got, want in zip((bank.w_up.grad, bank.w_gate.grad, bank.w_down.grad), gw3):
+            assert rel_l2(got, want) < TOL
+        empty = plan.counts == 0
+        assert (bank.w_up.grad.cpu()[empty] == 0).all() and (bank.w_down.grad.cpu()[empty] == 0).all()
+        if kept is not None:
+            dropped = (kept == 0).view(tokens, slots)
+            assert (tw.grad.cpu()[dropped] == 0).all()
+
+
+@pytest.mark.parametrize("workload,seeds", [("mlp_200m", (0, 1, 2)), ("mlp_1b", (0,))])
+def test_full_size_pool_step_vs_gold_on_gpu(cuda, workload, seeds):
+    """The 200m-like and 1b-like configs at full size.  The gold here is the same
+    oracle code run on the GPU in fp32 (a CPU pass of 1.5e13 FLOP would take
+    minutes), fed the routing the HIP path chose."""
+
+    from nestor_amd.workloads import WORKLOADS, build_pool, expert_mlp_step, make_tensors
+
+    w = WORKLOADS[workload]
+    for seed in seeds:
+        t = make_tensors(w, seed, cuda)
+        column_router, pool = build_pool(w, t)
+        x = t.x.clone().requires_grad_(True)
+        captured = {}
+        orig = pool._bank
+
+        def spy(flat_x, experts, stacked, ids, weights, group, _orig=orig):
+            out = _orig(flat_x, experts, stacked, ids, weights, group)
+            captured[stacked] = (ids.detach(), weights, group, out)
+            return out
+
+        pool._bank = spy
+        update = expert_mlp_step(w, column_router, pool, x, t.grad_out)
+        assert update.shape == (1, w.tokens, w.d_model)
+        # Each bank call against the fp32 gold on identical routing.
+        for stacked, w3 in ((pool.stacked_public, t.pub), (pool.stacked_private, t.priv)):
+            ids, weights, group, out = captured[stacked]
+            xs = t.x.float()
+            ref = obank.gold_combine(xs, *[b.float() for b in w3], ids, weights.detach().float(), group)
+            assert rel_l2(out, ref) < TOL, (workload, seed)
+            counts = torch.bincount(ids.reshape(-1), minlength=stacked.num_experts)
+            assert int(counts.sum()) == ids.numel()
+            del ref
+        # Gradients of the whole step: fp32 autograd through the gold with the same routing.
+        xs = t.x.float().requires_grad_(True)
+        gold_params = []
+        total = 0
+        alpha = torch.softmax((xs.detach() @ pool.path_gate.weight.float().t()), -1).to(torch.bfloat16).float()
+        for k, (stacked, w3) in enumerate(((pool.stacked_public, t.pub), (pool.stacked_private, t.priv))):
+            ids, weights, group, _ = captured[stacked]
+            w3f = [b.float().requires_grad_(True) for b in w3]
+            gold_params.append(w3f)
+            part = obank.gold_combine(xs, *w3f, ids, weights.detach().float(), ids.shape[1])
+            total = total + alpha[:, k:k + 1] * part.reshape(w.tokens, w.d_model)
+        total.backward(t.grad_out.float())
+        for (stacked, _), w3f in zip(((pool.stacked_public, t.pub), (pool.stacked_private, t.priv)), gold_params):
+            for got, want, n in zip((stacked.w_up.grad, stacked.w_gate.grad, stacked.w_down.grad), w3f,
+                                    ("w_up", "w_gate", "w_down")):
+                assert rel_l2(got, want.grad) < 1.5e-2, (workload, seed, n)
+        del gold_params, total, xs, t, pool, captured
+        torch.cuda.empty_cache()

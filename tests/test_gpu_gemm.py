@@ -84,7 +84,7 @@ def test_upgate_swiglu_fused_matches_unfused(cuda, tokens, slots, banks, K, H, s
     tu = w_up.to(cuda).requires_grad_(True)
     tg = w_gate.to(cuda).requires_grad_(True)
     up_gate, hidden = ops.upgate_swiglu_op(tx, tu, tg, got.tile_table, got.offs,
-                                           got.padded_starts, got.counts)
+                                           got.padded_starts, got.kept_counts)
     torch.testing.assert_close(up_gate.cpu().float(), ug_ref.float(), rtol=2 ** -6, atol=1e-3)
     torch.testing.assert_close(hidden.cpu().float(), hid_ref.float(), rtol=2 ** -5, atol=2e-3)
     assert rel_l2(hidden, hid_ref) < 3e-3

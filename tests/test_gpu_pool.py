@@ -1,0 +1,111 @@
+"""ExpertPoolMLP on the HIP path: the three output layouts agree with each other
+and with the per-token definition of the pool equation."""
+
+import pytest
+import torch
+
+from tests.helpers import gen, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _pool(cuda, stacked: bool):
+    import nestor_amd as na
+
+    torch.manual_seed(9)
+    pool = na.ExpertPoolMLP(
+        dim=40, num_groups=4, num_groups_per_token=2, num_public_experts=4, public_top_k=2,
+        num_private_experts=3, private_top_k=2, router_score_mlp_hidden_dims=[],
+        private_gate_mode="switch",
+    )
+    with torch.no_grad():
+        pool.path_gate.weight.normal_()
+        for r in [pool.public_router, *pool.private_routers]:
+            r.choice_bias.normal_(std=0.1)
+    if stacked:
+        assert na.consolidate_stacked_expert_banks(pool, force=True) == 2
+    pool.triton_fused = pool.triton_index = pool.fused_gate = True
+    return pool.to(cuda).eval()
+
+
+def _inputs(cuda):
+    g = gen(21)
+    x = torch.randn(3, 70, 40, generator=g)
+    valid = torch.ones(3, 70, dtype=torch.bool)
+    valid[1, -5:] = False
+    scores = torch.rand(3, 70, 4, generator=g)
+    slot_groups = scores.topk(2, dim=-1).indices
+    active = torch.zeros(3, 70, 4, dtype=torch.bool).scatter(-1, slot_groups, True) & valid.unsqueeze(-1)
+    gates = torch.zeros(3, 70, 4).scatter(-1, slot_groups, 0.5) * valid.unsqueeze(-1)
+    return tuple(t.to(cuda) for t in (x, valid, gates, active, slot_groups))
+
+
+def _per_token_reference(pool, x, valid, gates, active):
+    """The pool equation token by token in fp32, on the routing the pool chose
+    (the slow-loop form of the reference's tests/test_expert_pools.py:126-180)."""
+
+    out = torch.zeros_like(x)
+    B, S, _ = x.shape
+
+    def routed(router, experts, h, ok):
+        if not ok:
+            return torch.zeros_like(h)
+        r = router(h.view(1, 1, -1), torch.ones(1, 1, dtype=torch.bool, device=h.device))
+        acc = torch.zeros_like(h)
+        for e in r.topk_indices.view(-1).tolist():
+            acc = acc + r.gates.view(-1)[e] * experts[e](h)
+        return acc
+
+    for b in range(B):
+        for s in range(S):
+            h = x[b, s]
+            alpha = torch.softmax(pool.path_gate(h).float(), -1)
+            pub = routed(pool.public_router, pool.public_experts, h, bool(valid[b, s]))
+            priv = torch.zeros_like(h)
+            for g in range(pool.num_groups):
+                if active[b, s, g] and valid[b, s]:
+                    priv = priv + gates[b, s, g] * routed(pool.private_routers[g], pool.private_experts[g], h, True)
+            out[b, s] = alpha[0] * pub + alpha[1] * priv
+    return out
+
+
+@pytest.mark.parametrize("stacked", [True, False])
+def test_pool_layouts_and_definition(cuda, stacked):
+    pool = _pool(cuda, stacked)
+    x, valid, gates, active, slot_groups = _inputs(cuda)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        summed, pub_out, priv_outs = pool(x, valid, gates, active)
+        p_slot, v_slot, _, _ = pool.forward_per_slot(x, valid, gates, active, slot_groups)
+        p_grp, v_grp, _, _ = pool.forward_per_group(x, valid, gates, active)
+    assert summed.dtype == torch.float32 and v_slot.shape == (3, 70, 2, 40) and v_grp.shape == (3, 70, 4, 40)
+    assert len(priv_outs) == 4 and torch.equal(pub_out.valid_token_mask, valid)
+    for gi, po in enumerate(priv_outs):
+        assert torch.equal(po.valid_token_mask, valid & active[:, :, gi])
+    # layouts: public + private summed over slots / groups == the summed forward
+    torch.testing.assert_close(p_slot + v_slot.sum(2), summed, rtol=2 ** -6, atol=1e-2)
+    torch.testing.assert_close(p_grp + v_grp.sum(2), summed, rtol=2 ** -6, atol=1e-2)
+    idx = slot_groups.unsqueeze(-1).expand(-1, -1, -1, 40)
+    torch.testing.assert_close(v_grp.gather(2, idx), v_slot, rtol=2 ** -6, atol=1e-2)
+    # definition: per-token loop in fp32 with torch ops only
+    with torch.no_grad():
+        ref = _per_token_reference(pool, x, valid, gates, active)
+    assert rel_l2(summed, ref) < 1e-2
+    assert (summed[~valid] == 0).all()
+
+
+def test_pool_grads_reach_every_parameter(cuda):
+    """Every parameter ends a step with a finite gradient, including banks no
+    token selected (the reference's DDP-safety property,
+    tests/test_expert_pools.py:428-436)."""
+
+    pool = _pool(cuda, True).train()
+    x, valid, gates, active, slot_groups = _inputs(cuda)
+    x = x.requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        pub, priv, _, _ = pool.forward_per_slot(x, valid, gates, active, slot_groups)
+    (pub.float().sum() + priv.float().square().sum()).backward()
+    names = [n for n, _ in pool.named_parameters()]
+    assert "stacked_public.w_up" in names and "stacked_private.w_down" in names
+    for n, p in pool.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all(), n
+    assert x.grad is not None and torch.isfinite(x.grad).all()

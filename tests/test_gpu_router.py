@@ -1,0 +1,102 @@
+"""Router epilogue kernel and slot construction vs the oracle: indices and ids
+bit-exact, probabilities / gates to fp32 or one-bf16-ulp accuracy."""
+
+import pytest
+import torch
+
+from oracle import router as orouter
+from tests.helpers import gen
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,choices,k,mode", [
+    (1000, 8, 2, "renorm"), (1000, 4, 1, "renorm"), (4096, 16, 1, "switch"), (777, 15, 2, "switch"),
+    (513, 32, 2, "renorm"), (100, 64, 8, "renorm"), (64, 1, 1, "renorm"), (300, 12, 3, "switch"),
+])
+def test_router_topk_kernel(cuda, dtype, n, choices, k, mode):
+    from nestor_amd import ops
+
+    g = gen(n + choices)
+    scores = torch.randn(n, choices, generator=g).to(dtype)  # bf16 scores tie often
+    bias = torch.randn(choices, generator=g) * 0.1
+    mask = torch.rand(n, generator=g) > 0.1
+    want = orouter.route(scores, bias, k, mode, mask, softmax_dtype=torch.float32)
+    probs, topk, gates = ops.router_topk(scores.to(cuda), bias.to(cuda).view(1, -1), mask.to(cuda), k,
+                                         1 if mode == "switch" else 0)
+    assert torch.equal(topk.cpu(), want.topk_indices)  # ties: lowest index first on both sides
+    torch.testing.assert_close(probs.cpu(), want.softmax_probs, rtol=1e-5, atol=1e-7)
+    assert gates.dtype == dtype
+    if dtype == torch.float32:
+        torch.testing.assert_close(gates.cpu(), want.gates, rtol=1e-5, atol=1e-7)
+    else:
+        torch.testing.assert_close(gates.cpu().float(), want.gates.float(), rtol=2 ** -7, atol=1e-6)
+    assert torch.equal(gates.cpu() > 0, want.active_mask) or dtype == torch.bfloat16
+    assert (gates.cpu()[~mask] == 0).all()
+    if k == 1 and mode == "renorm":
+        # closed form: a renormalised top-1 gate is exactly 1 on valid tokens
+        assert torch.equal(gates.cpu().float().sum(-1), mask.float())
+
+
+def test_batched_private_routers_and_slots(cuda):
+    """[T, G, Q] scores through one launch == G separate routers; slot ids are
+    ``column * Q + expert`` and weights ``private_gate * column_gate``."""
+
+    from nestor_amd import ops
+
+    tokens, groups, q, k_a = 2000, 8, 4, 2
+    g = gen(11)
+    scores = torch.randn(tokens, groups, q, generator=g).bfloat16()
+    bias = torch.randn(groups, q, generator=g) * 0.05
+    col_scores = torch.randn(tokens, groups, generator=g).bfloat16()
+    valid = torch.rand(tokens, generator=g) > 0.05
+    col = orouter.route(col_scores, torch.zeros(groups), k_a, "renorm", valid)
+    want = orouter.route_private_batched(
+        scores.view(1, tokens, groups, q), bias, 1, "switch", valid.view(1, tokens),
+        col.active_mask.view(1, tokens, groups), softmax_dtype=torch.float32,
+    )
+    member = (valid.unsqueeze(-1) & col.active_mask).reshape(-1)
+    probs, topk, gates = ops.router_topk(
+        scores.view(-1, q).to(cuda), bias.to(cuda), member.to(cuda), 1, 1)
+    assert torch.equal(topk.cpu().view(1, tokens, groups, 1), want.topk_indices)
+    torch.testing.assert_close(gates.cpu().float().view(1, tokens, groups, q),
+                               want.gates.float(), rtol=2 ** -7, atol=1e-6)
+    # per-router loop pins the batched oracle itself
+    for gi in range(groups):
+        one = orouter.route(scores[:, gi], bias[gi], 1, "switch", valid & col.active_mask[:, gi])
+        assert torch.equal(one.topk_indices, want.topk_indices[0, :, gi])
+        assert torch.equal(one.gates, want.gates[0, :, gi])
+
+
+def test_pool_routing_matches_oracle_slots(cuda):
+    """Pool routers + slot build on the GPU vs the oracle on the same scores."""
+
+    from nestor_amd.workloads import WORKLOADS, build_pool, make_tensors
+
+    w = WORKLOADS["tiny_100m"]
+    t = make_tensors(w, 0, cuda)
+    column_router, pool = build_pool(w, t)
+    x3 = t.x.view(1, w.tokens, w.d_model)
+    valid = torch.ones(1, w.tokens, dtype=torch.bool, device=cuda)
+    with torch.no_grad():
+        col = column_router(x3, valid)
+        pub, privs, stacked = pool._route(x3, valid, col.active_mask)
+        ids, weights, selected = pool._private_slots(
+            privs, col.gates.view(w.tokens, -1), w.tokens,
+            selected=col.topk_indices.view(w.tokens, -1), stacked=stacked)
+        pub_ids, pub_w = pool._public_slots(pub, w.tokens)
+    # oracle on the scores the GPU produced (score GEMMs are plain library GEMMs)
+    ocol = orouter.route(col.scores.cpu()[0], torch.zeros(w.columns), 2, "renorm", valid.cpu()[0])
+    assert torch.equal(col.topk_indices.cpu()[0], ocol.topk_indices)
+    torch.testing.assert_close(col.gates.cpu()[0].float(), ocol.gates.float(), rtol=2 ** -7, atol=1e-6)
+    pscores = torch.stack([p.scores for p in privs], dim=-2).cpu()
+    opriv = orouter.route_private_batched(
+        pscores, torch.zeros(w.columns, w.private), 1, "switch", valid.cpu(), ocol.active_mask.unsqueeze(0))
+    oids, ow, _ = orouter.private_slots(
+        opriv.gates[0], opriv.topk_indices[0], ocol.gates, 2, selected=ocol.topk_indices)
+    assert torch.equal(ids.cpu(), oids)  # token -> column -> expert ids: exact
+    torch.testing.assert_close(weights.cpu().float(), ow.float(), rtol=2 ** -6, atol=1e-6)
+    opub = orouter.route(pub.scores.cpu()[0], torch.zeros(w.public), 1, "renorm", valid.cpu()[0])
+    assert torch.equal(pub_ids.cpu(), opub.topk_indices)
+    assert torch.equal(pub_w.cpu().float(), torch.ones(w.tokens, 1))
