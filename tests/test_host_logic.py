@@ -1,0 +1,128 @@
+"""Host-side pieces that need no GPU: stacked layout, width contract, flags,
+and loud failure of the product path off-GPU."""
+
+import os
+
+import pytest
+import torch
+
+import nestor_amd as na
+from nestor_amd import flags
+from nestor_amd.pool import private_expert_hidden_dim, public_expert_hidden_dim
+
+
+def test_width_contract_table():
+    """The reference's documented widths (tests/test_expert_pools.py:186-215)."""
+
+    assert public_expert_hidden_dim(640, 1) == 1280
+    assert private_expert_hidden_dim(640, 3, 1) == 424
+    assert public_expert_hidden_dim(960, 1) == 1920
+    assert private_expert_hidden_dim(960, 3, 1) == 640
+    assert public_expert_hidden_dim(1280, 1) == 2560
+    assert private_expert_hidden_dim(1280, 3, 1) == 856
+    assert public_expert_hidden_dim(640, 2) == 640
+    assert private_expert_hidden_dim(640, 3, 2) == 216
+    assert public_expert_hidden_dim(640, 2, active_budget=1.25) == 400
+    assert private_expert_hidden_dim(640, 8, 1, active_budget=1.25) == 96
+    assert private_expert_hidden_dim(640, 3, 1, with_public_pool=False) == 856
+    # the measurement configs: active_budget 4 makes private == public == 2d
+    assert private_expert_hidden_dim(2048, 2, 1, active_budget=4.0) == 4096
+    assert public_expert_hidden_dim(2048, 1) == 4096
+
+
+def test_stacked_bank_layout_and_views():
+    """w_up[i].t() is expert i's up weight; per-expert params leave the module
+    tree; state-dict keys are the stacked ones
+    (tests/test_stacked_expert_banks.py:87-101,198-200 in the reference)."""
+
+    torch.manual_seed(0)
+    experts = [na.SwigluExpert(12, 20, 12) for _ in range(3)]
+    before = [(e.layers[0].weight.detach().clone(), e.gate.weight.detach().clone(),
+               e.layers[1].weight.detach().clone()) for e in experts]
+    bank = na.StackedExpertBank(experts)
+    assert bank.w_up.shape == (3, 12, 20) and bank.w_gate.shape == (3, 12, 20)
+    assert bank.w_down.shape == (3, 20, 12) and bank.w_up.is_contiguous()
+    for i, (up, gate, down) in enumerate(before):
+        assert torch.equal(bank.w_up[i].t(), up) and torch.equal(bank.w_gate[i].t(), gate)
+        assert torch.equal(bank.w_down[i].t(), down)
+        assert experts[i].layers[0].weight.data_ptr() == bank.w_up[i].data_ptr()
+    assert all(len(list(e.parameters())) == 0 for e in experts)
+    x = torch.randn(5, 12)
+    ref = torch.nn.functional.silu(x @ before[1][1].t()) * (x @ before[1][0].t()) @ before[1][2].t()
+    torch.testing.assert_close(experts[1](x), ref)
+    experts[1](x).sum().backward()
+    assert bank.w_up.grad is not None and (bank.w_up.grad[0] == 0).all() and bank.w_up.grad[1].abs().sum() > 0
+
+    pool = na.ExpertPoolMLP(16, 2, 1, 2, 1, 2, 1, [])
+    assert na.consolidate_stacked_expert_banks(pool) == 0  # flag unset
+    assert na.consolidate_stacked_expert_banks(pool, force=True) == 2
+    keys = pool.state_dict().keys()
+    for k in ("stacked_public.w_up", "stacked_public.w_gate", "stacked_public.w_down",
+              "stacked_private.w_up", "stacked_private.w_down"):
+        assert k in keys
+    assert not any("public_experts" in k or "private_experts" in k for k in keys)
+    assert pool.stacked_private.w_up.shape == (4, 16, private_expert_hidden_dim(16, 1, 1))
+    moved = pool.to(torch.float64)
+    first = moved._private_bank()[0]
+    assert first.layers[0].weight.dtype == torch.float64
+    assert first.layers[0].weight.data_ptr() == moved.stacked_private.w_up.data_ptr()
+
+
+def test_non_uniform_bank_is_rejected():
+    a, b = na.SwigluExpert(8, 8, 8), na.SwigluExpert(8, 8, 8, bias=True)
+    with pytest.raises(ValueError):
+        na.StackedExpertBank([a, b])
+    with pytest.raises(ValueError):
+        na.ExpertPoolMLP(16, 2, 3, 2, 1, 2, 1, [])
+    with pytest.raises(ValueError):
+        na.ExpertPoolMLP(16, 2, 1, 2, 1, 0, 1, [])
+
+
+def test_flag_readers_follow_env():
+    saved = {k: os.environ.get(k) for k in (
+        "NESTOR_TRITON_INDEX_BUILD", "NESTOR_TRITON_EXPERT_DISPATCH", "NESTOR_STACKED_EXPERT_BANKS",
+        "NESTOR_GROUPED_MM_FUSED_GATE", "NESTOR_TRITON_EXPERT_CATCAST", "NESTOR_BATCHED_ROUTERS")}
+    try:
+        for k in saved:
+            os.environ.pop(k, None)
+        assert not flags.triton_index_requested() and not flags.triton_expert_requested()
+        assert not flags.stacked_banks_requested() and not flags.fused_gate_requested()
+        assert flags.triton_cat_cast_requested() and not flags.batched_routers_enabled()
+        os.environ["NESTOR_TRITON_INDEX_BUILD"] = "1"
+        assert flags.triton_index_requested() and flags.triton_expert_requested()  # default follows
+        os.environ["NESTOR_TRITON_EXPERT_DISPATCH"] = "0"
+        assert not flags.triton_expert_requested()
+        os.environ["NESTOR_STACKED_EXPERT_BANKS"] = "1"
+        assert flags.stacked_banks_requested()
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+
+
+def test_product_path_refuses_cpu_tensors():
+    """No CPU fallback: calling the path with CPU tensors raises instead of
+    silently computing somewhere else."""
+
+    bank = na.StackedExpertBank.from_tensors(
+        torch.randn(2, 8, 16).bfloat16(), torch.randn(2, 8, 16).bfloat16(), torch.randn(2, 16, 8).bfloat16())
+    x = torch.randn(4, 8).bfloat16()
+    ids = torch.zeros(4, 1, dtype=torch.long)
+    w = torch.ones(4, 1)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        na.grouped_expert_combine(x, bank.expert_views(), ids, w, 1, stacked=bank, triton_fused=True)
+    with pytest.raises(NotImplementedError):
+        na.grouped_expert_combine(x.float(), bank.expert_views(), ids, w, 1, stacked=bank)  # fp32 GEMM dtype
+
+
+def test_workload_flop_convention():
+    from nestor_amd.workloads import WORKLOADS
+
+    w = WORKLOADS["mlp_1b"]
+    assert w.experts == 144 and w.assignments == 3
+    assert w.gemm_flops(False) == pytest.approx(4.948e12, rel=1e-3)
+    assert w.gemm_flops(True) == pytest.approx(1.4843e13, rel=1e-3)
+    assert WORKLOADS["tiny_100m"].gemm_flops() == pytest.approx(3.866e10, rel=1e-3)
+    assert WORKLOADS["mlp_200m"].gemm_flops(True) == pytest.approx(1.855e12, rel=1e-3)

@@ -1,0 +1,48 @@
+"""The C-ABI library loads and exports every entry point the header declares
+(no compute: runs without a GPU)."""
+
+import ctypes
+import os
+import re
+
+from nestor_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared() -> list[str]:
+    text = open(os.path.join(ROOT, "include", "nestor_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nestor_hip_\w+)\s*\(", text)))
+
+
+def test_header_symbols_exported_and_bound():
+    names = _declared()
+    assert len(names) >= 22
+    assert _lib.LIB_PATH.exists(), "build the library first: python -m nestor_amd.build"
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert sorted(_lib.EXPORTED_SYMBOLS) == names, "ctypes table and header disagree"
+
+
+def test_version_and_error_strings():
+    lib = _lib.load()
+    assert lib.nestor_hip_abi_version() == _lib.ABI_VERSION
+    assert lib.nestor_hip_strerror(0) == b"ok"
+    assert b"invalid" in lib.nestor_hip_strerror(-22)
+    assert lib.nestor_hip_max_tiles(67584, 128) == 67584 // 128 + 128 + 2
+    assert lib.nestor_hip_index_build_workspace_bytes(65536, 128) == 128 * 128 * 4
+
+
+def test_argument_checks_fail_before_any_launch():
+    """Bad sizes are rejected with EINVAL on the host (null pointers, no GPU needed)."""
+
+    lib = _lib.load()
+    null = ctypes.c_void_p(0)
+    assert lib.nestor_hip_dispatch_rows_fwd(null, 1, null, null, 1, null, 16, 12, null) == -22  # dim % 8
+    assert lib.nestor_hip_swiglu_fwd(null, null, null, 4, 20, 20, 20, null) == -22
+    assert lib.nestor_hip_grouped_gemm_nn(null, null, null, 16, 12, 8, 1, null, 4, null) == -22
+    assert lib.nestor_hip_router_topk(null, 1, null, 1, null, null, null, null, 4, 65, 1, 0, null) == -22
+    assert lib.nestor_hip_index_build(null, 10, 5000, 1, 0, 0, 1, null, null, null, null, null, null,
+                                      null, null, null, null, null, null, 0, null, 0, null) == -34
