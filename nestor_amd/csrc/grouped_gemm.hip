@@ -1,11 +1,11 @@
 // Grouped expert GEMMs on the gfx950 matrix cores.
 //
-// One workgroup (4 wavefronts, 2 x 2) owns a 128 x 128 output tile and walks K
-// in steps of 64 through double-buffered LDS; each wavefront keeps a 64 x 64
-// accumulator as 2 x 2 v_mfma_f32_32x32x16_bf16 tiles.  Which rows form a tile
-// and which bank multiplies them comes from the device-side tile table written
-// by the index build, so no launch parameter depends on the routing and the
-// host never reads a count.
+// A workgroup of 4 wavefronts owns a BM x BN output tile and walks the
+// contraction in steps of BK through double-buffered LDS; each wavefront keeps
+// a (BM / WGM) x (BN / WGN) accumulator as v_mfma_f32_32x32x16_bf16 tiles.
+// Which rows form a tile and which bank multiplies them comes from the
+// device-side tile table written by the index build, so no launch parameter
+// depends on the routing and the host never reads a count.
 //
 // Operand tiles sit in LDS in the layout they have in HBM.  An operand whose
 // contraction index is contiguous in memory (activations in the forward and
@@ -18,30 +18,52 @@
 // indices for one output index -- the MFMA operand layout, with no transpose
 // pass over the weights or activations in HBM.
 //
+// Software pipeline per K step: the tile for step t+1 goes from registers to
+// the idle LDS buffer, the global loads for step t+2 are issued, then step t is
+// computed from the other buffer with MFMA operand fragments double-buffered in
+// registers, so global latency hides behind a whole K step and LDS latency
+// behind the previous fragment's MFMAs.
+//
 // The MFMA is issued with its operands swapped (B fragment first), which
 // produces the transposed 32 x 32 tile: every lane then holds four consecutive
 // output columns of one row and the epilogue can stage the bf16 tile through
 // LDS with 64-bit writes and leave through 128-bit coalesced stores.
+#include <cstdlib>
+#include <type_traits>
+#include <utility>
+
 #include "common.hpp"
 
 namespace nestor {
 namespace {
 
-constexpr int BM = 128;
-constexpr int BN = 128;
-constexpr int BK = 64;
 constexpr int kThreads = 256;
-constexpr int KC_LD = BK + 8;    // row stride (elements) of a contraction-contiguous tile
-constexpr int NC_LD = BN + 16;   // row stride of a contraction-major tile
-constexpr int TILE_ELEMS = BM * KC_LD;  // == BK * NC_LD == 9216
-static_assert(BM * KC_LD == BK * NC_LD, "both tile layouts share one buffer size");
-constexpr int STAGE_LD = BN + 8;
-constexpr size_t kGemmLds = 4 * TILE_ELEMS * sizeof(uint16_t);  // 2 stages x (A, B)
-static_assert(BM * STAGE_LD <= 2 * TILE_ELEMS, "epilogue staging reuses the A buffers");
-static_assert(NESTOR_HIP_TILE_M == BM, "tile table granularity");
+constexpr int kWaves = kThreads / kWave;
 
 #define NESTOR_LDS __attribute__((address_space(3)))
-typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
+struct Cfg {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
+  static_assert(WGM * WGN == kWaves, "4 wavefronts per workgroup");
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;  // wavefront tile
+  static constexpr int MI = WTM / 32, NJ = WTN / 32;    // MFMA tiles per wavefront
+  static constexpr int KK = BK / 16;
+  static constexpr int KC_LD = BK + 8;       // row stride of a contraction-contiguous tile
+  static constexpr int STAGE_LD = BN + 8;    // epilogue staging row stride
+  // Tile sizes in elements for the two layouts of each operand.
+  static constexpr int A_KC = BM * KC_LD, A_MC = BK * (BM + 16);
+  static constexpr int B_KC = BN * KC_LD, B_NC = BK * (BN + 16);
+  static constexpr int A_ELEMS = A_KC > A_MC ? A_KC : A_MC;
+  static constexpr int B_ELEMS = B_KC > B_NC ? B_KC : B_NC;
+  static constexpr int STAGE_ELEMS = BM * STAGE_LD;
+  static constexpr int PIPE_ELEMS = 2 * (A_ELEMS + B_ELEMS);
+  static constexpr size_t LDS_BYTES =
+      sizeof(uint16_t) * (PIPE_ELEMS > STAGE_ELEMS ? PIPE_ELEMS : STAGE_ELEMS);
+  static constexpr int A_CHUNKS = BM * BK / 8 / kThreads;  // 16-byte chunks per thread
+  static constexpr int B_CHUNKS = BN * BK / 8 / kThreads;
+  static_assert(BM * BK / 8 % kThreads == 0 && BN * BK / 8 % kThreads == 0, "chunking");
+};
 
 enum GemmMode {
   kNN = 0,        // out = a @ b[bank]            b [E,K,N]
@@ -49,6 +71,7 @@ enum GemmMode {
   kNT = 2,        // out = a @ b[bank]^T          b [E,N,K]
   kNTUpGate = 3,  // out = g[:, :H] @ w_up^T + g[:, H:] @ w_gate^T
   kNNFp8W = 4,    // kNN with e4m3 weights and per-column scales
+  kTN = 5,        // out[bank] = a[seg]^T @ g[seg]   (weight gradient)
 };
 
 struct GemmParams {
@@ -56,30 +79,38 @@ struct GemmParams {
   int64_t lda;
   const void* b0;
   const void* b1;
-  int64_t bank_stride;  // elements between banks of b0 / b1
+  int64_t bank_stride;  // elements between banks of b0 / b1 (kTN: of out)
   int64_t ldb;
   const float* scale;   // [E, N] (kNNFp8W)
   uint16_t* out;
   int64_t ldo;
   uint16_t* out2;       // hidden (kNNUpGate)
   int64_t ldo2;
-  int64_t K;            // contraction length (per phase)
+  int64_t K;            // contraction length (per phase); kTN: unused
   int64_t N;            // output columns (kNNUpGate: H)
+  int64_t M;            // kTN: output rows
   const int32_t* tile_table;
   int64_t max_tiles;
   int n_tiles;
+  // kTN segment description
+  int64_t rows_pad;
+  const int32_t* offs;
+  const int64_t* seg_start;
+  const int64_t* seg_count;
 };
 
+template <int LD>
 __device__ __forceinline__ bf16x8 lds_read_kc(const uint16_t* tile, int row, int k) {
-  return *reinterpret_cast<const bf16x8*>(tile + row * KC_LD + k);
+  return *reinterpret_cast<const bf16x8*>(tile + row * LD + k);
 }
 
-// Eight consecutive contraction indices (k .. k+7) of output index `col`, from
-// a contraction-major tile, as two transposing 64-bit LDS reads.
+// Eight consecutive contraction indices (krow .. krow+7 of this lane's half) of
+// output index `col`, from a contraction-major tile, as two transposing reads.
+template <int LD>
 __device__ __forceinline__ bf16x8 lds_read_tr(const uint16_t* tile, int krow, int col) {
   typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
-  const uint16_t* p0 = tile + krow * NC_LD + col;
-  const uint16_t* p1 = p0 + 4 * NC_LD;
+  const uint16_t* p0 = tile + krow * LD + col;
+  const uint16_t* p1 = p0 + 4 * LD;
   v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(p0));
   v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(p1));
   typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -101,222 +132,399 @@ __device__ __forceinline__ u32x4 fp8x8_to_bf16x8(u32x2 raw) {
   return pack8(f);
 }
 
-struct TileRef {
-  int bank;
-  int row0;
-  int nrows;
-};
-
-__device__ __forceinline__ bool fetch_tile(const int32_t* tt, int64_t max_tiles, int tile,
-                                           TileRef* t) {
-  if (tile >= tt[3 * max_tiles]) return false;
-  t->bank = tt[tile];
-  t->row0 = tt[max_tiles + tile];
-  t->nrows = tt[2 * max_tiles + tile];
-  return true;
+// Scheduling recipe for one fragment's worth of MFMAs: before MFMA m, let
+// through this MFMA's share of the LDS reads (0x100), LDS writes (0x200) and
+// global loads (0x020) that sit in the same scheduling region, so each memory
+// latency hides behind the matrix pipe (0x008) instead of in front of it.
+template <int kReads, int kWrites, int kVmem, int kMfma, int... Ms>
+__device__ __forceinline__ void interleave_memory(std::integer_sequence<int, Ms...>) {
+  (([] {
+     constexpr int m = Ms;
+     constexpr int r = ((m + 1) * kReads) / kMfma - (m * kReads) / kMfma;
+     constexpr int w = ((m + 1) * kWrites) / kMfma - (m * kWrites) / kMfma;
+     constexpr int v = ((m + 1) * kVmem) / kMfma - (m * kVmem) / kMfma;
+     if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+     if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);
+     if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
+     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+   }()),
+   ...);
 }
 
-// Accumulators -> bf16 staging tile [BM][STAGE_LD] (optionally scaled per column).
-template <bool kScale>
-__device__ __forceinline__ void stage_accumulators(uint16_t* stage, const f32x16 (&acc)[2][2],
-                                                   int wm, int wn, int lane,
-                                                   const float* col_scale, int64_t n0,
-                                                   int64_t n_limit) {
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int m = 64 * wm + 32 * i + (lane & 31);
-        const int n = 64 * wn + 32 * j + 8 * q + 4 * (lane >> 5);
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
-        if constexpr (kScale) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            v[e] *= (n0 + n + e < n_limit) ? col_scale[n0 + n + e] : 0.0f;
-        }
-        u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        *reinterpret_cast<u32x2*>(stage + m * STAGE_LD + n) = packed;
-      }
-}
-
-template <int kMode>
+template <typename C, int kMode>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   extern __shared__ __align__(16) uint16_t lds[];
+  constexpr int BM = C::BM, BN = C::BN, BK = C::BK;
+  constexpr bool kUpGateFwd = kMode == kNNUpGate;
+  constexpr bool kAContig = kMode != kTN;                         // a is [rows, K]
+  constexpr bool kBContig = kMode == kNT || kMode == kNTUpGate;   // b is [N, K]
+  constexpr int kOutCols = kUpGateFwd ? BN / 2 : BN;              // output columns per tile
+  constexpr int A_LD = kAContig ? C::KC_LD : BM + 16;
+  constexpr int B_LD = kBContig ? C::KC_LD : BN + 16;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1;
-  const int wn = wave & 1;
-  const int tile = blockIdx.x / p.n_tiles;
-  const int nt = blockIdx.x % p.n_tiles;
-  TileRef t;
-  if (!fetch_tile(p.tile_table, p.max_tiles, tile, &t)) return;
+  const int wm = wave / C::WGN;
+  const int wn = wave % C::WGN;
 
-  constexpr bool kUpGateFwd = kMode == kNNUpGate;
-  constexpr bool kBContig = kMode == kNT || kMode == kNTUpGate;  // b is [N, K]
-  constexpr int kOutCols = kUpGateFwd ? BN / 2 : BN;  // output columns per tile
-  const int64_t n0 = static_cast<int64_t>(nt) * kOutCols;
-
-  if (t.bank < 0) {
-    // Slack tail: every padded tensor holds zeros there.
-    const u32x4 zero = {0, 0, 0, 0};
-    for (int c = tid; c < BM * (kOutCols / 8); c += kThreads) {
-      const int row = c / (kOutCols / 8);
-      const int64_t n = n0 + (c % (kOutCols / 8)) * 8;
-      if (row < t.nrows && n < p.N) {
-        const int64_t r = t.row0 + row;
-        if constexpr (kUpGateFwd) {
-          if (p.out != nullptr) {
+  // ---- which tile -------------------------------------------------------
+  int bank, row0 = 0, nrows = BM;
+  int64_t n0, m0 = 0;
+  int64_t seg_begin = 0, seg_end = 0;
+  if constexpr (kMode == kTN) {
+    bank = blockIdx.z;
+    m0 = static_cast<int64_t>(blockIdx.y) * BM;
+    n0 = static_cast<int64_t>(blockIdx.x) * BN;
+    if (p.seg_start != nullptr) {
+      seg_begin = p.seg_start[bank];
+      seg_end = seg_begin + p.seg_count[bank];
+    } else {
+      seg_begin = bank == 0 ? 0 : p.offs[bank - 1];
+      seg_end = p.offs[bank];
+    }
+    if (seg_end > p.rows_pad) seg_end = p.rows_pad;
+  } else {
+    const int tile = blockIdx.x / p.n_tiles;
+    const int nt = blockIdx.x % p.n_tiles;
+    const int32_t* tt = p.tile_table;
+    if (tile >= tt[3 * p.max_tiles]) return;
+    bank = tt[tile];
+    row0 = tt[p.max_tiles + tile];
+    nrows = tt[2 * p.max_tiles + tile];
+    n0 = static_cast<int64_t>(nt) * kOutCols;
+    if (bank < 0) {
+      // Slack tail: every padded tensor holds zeros there.
+      const u32x4 zero = {0, 0, 0, 0};
+      for (int c = tid; c < BM * (kOutCols / 8); c += kThreads) {
+        const int row = c / (kOutCols / 8);
+        const int64_t n = n0 + (c % (kOutCols / 8)) * 8;
+        if (row < nrows && n < p.N) {
+          const int64_t r = row0 + row;
+          if constexpr (kUpGateFwd) {
+            if (p.out != nullptr) {
+              st16(p.out + r * p.ldo + n, zero);
+              st16(p.out + r * p.ldo + p.N + n, zero);
+            }
+            st16(p.out2 + r * p.ldo2 + n, zero);
+          } else {
             st16(p.out + r * p.ldo + n, zero);
-            st16(p.out + r * p.ldo + p.N + n, zero);
           }
-          st16(p.out2 + r * p.ldo2 + n, zero);
+        }
+      }
+      return;
+    }
+  }
+
+  int num_kt, kt_per_phase = 1;
+  if constexpr (kMode == kTN) {
+    num_kt = seg_end > seg_begin ? static_cast<int>((seg_end - seg_begin + BK - 1) / BK) : 0;
+  } else {
+    kt_per_phase = static_cast<int>((p.K + BK - 1) / BK);
+    num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
+  }
+  const uint16_t* a_rows = p.a + static_cast<int64_t>(row0) * p.lda;
+
+  u32x4 ra[C::A_CHUNKS], rb[C::B_CHUNKS];
+  const u32x4 zero4 = {0, 0, 0, 0};
+
+  // Global -> register tile loads.  Every load is unconditional: indices that
+  // fall outside the tile are clamped to a valid element (their products only
+  // reach output rows / columns that are never stored), and only the partial
+  // last step of the contraction (kTail) zeroes what it must not sum.
+  bool has_tail;
+  if constexpr (kMode == kTN)
+    has_tail = ((seg_end - seg_begin) % BK) != 0;
+  else
+    has_tail = (p.K % BK) != 0;
+  const int last_row = nrows - 1;
+
+  auto load_a = [&](int kt, auto tail_tag) {
+    constexpr bool kTail = decltype(tail_tag)::value;
+    if constexpr (kAContig) {
+      const int phase = kMode == kNTUpGate ? kt / kt_per_phase : 0;
+      const int64_t k0 = static_cast<int64_t>(kt - phase * kt_per_phase) * BK;
+      const int64_t col0 = kMode == kNTUpGate ? phase * p.K : 0;
+#pragma unroll
+      for (int i = 0; i < C::A_CHUNKS; ++i) {
+        const int c = tid + kThreads * i;
+        int row = c / (BK / 8);
+        row = row < last_row ? row : last_row;
+        const int64_t k = k0 + (c % (BK / 8)) * 8;
+        if constexpr (kTail) {
+          const bool ok = k < p.K;
+          const u32x4 v = ld16(a_rows + row * p.lda + col0 + (ok ? k : 0));
+          ra[i] = ok ? v : zero4;
         } else {
-          st16(p.out + r * p.ldo + n, zero);
+          ra[i] = ld16(a_rows + row * p.lda + col0 + k);
+        }
+      }
+    } else {
+      const int64_t r0 = seg_begin + static_cast<int64_t>(kt) * BK;
+#pragma unroll
+      for (int i = 0; i < C::A_CHUNKS; ++i) {
+        const int c = tid + kThreads * i;
+        const int64_t r = r0 + c / (BM / 8);
+        int64_t m = m0 + (c % (BM / 8)) * 8;
+        m = m < p.M ? m : p.M - 8;
+        if constexpr (kTail) {
+          const bool ok = r < seg_end;
+          const u32x4 v = ld16(p.a + (ok ? r : seg_begin) * p.lda + m);
+          ra[i] = ok ? v : zero4;
+        } else {
+          ra[i] = ld16(p.a + r * p.lda + m);
         }
       }
     }
-    return;
-  }
-
-  const int kt_per_phase = static_cast<int>((p.K + BK - 1) / BK);
-  const int num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
-  const uint16_t* a_rows = p.a + static_cast<int64_t>(t.row0) * p.lda;
-
-  u32x4 ra[4], rb[4];
-  const u32x4 zero4 = {0, 0, 0, 0};
-
-  auto load_a = [&](int kt) {
-    const int phase = kMode == kNTUpGate ? kt / kt_per_phase : 0;
-    const int64_t k0 = static_cast<int64_t>(kt - phase * kt_per_phase) * BK;
-    const int64_t col0 = kMode == kNTUpGate ? phase * p.K : 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + kThreads * i;
-      const int row = c >> 3;
-      const int64_t k = k0 + (c & 7) * 8;
-      ra[i] = (row < t.nrows && k < p.K) ? ld16(a_rows + row * p.lda + col0 + k) : zero4;
-    }
   };
-  auto load_b = [&](int kt) {
-    if constexpr (kBContig) {
+  auto load_b = [&](int kt, auto tail_tag) {
+    constexpr bool kTail = decltype(tail_tag)::value;
+    if constexpr (kMode == kTN) {
+      const int64_t r0 = seg_begin + static_cast<int64_t>(kt) * BK;
+      const uint16_t* g = reinterpret_cast<const uint16_t*>(p.b0);
+#pragma unroll
+      for (int i = 0; i < C::B_CHUNKS; ++i) {
+        const int c = tid + kThreads * i;
+        const int64_t r = r0 + c / (BN / 8);
+        int64_t n = n0 + (c % (BN / 8)) * 8;
+        n = n < p.N ? n : p.N - 8;
+        if constexpr (kTail) {
+          const bool ok = r < seg_end;
+          const u32x4 v = ld16(g + (ok ? r : seg_begin) * p.ldb + n);
+          rb[i] = ok ? v : zero4;
+        } else {
+          rb[i] = ld16(g + r * p.ldb + n);
+        }
+      }
+    } else if constexpr (kBContig) {
       const int phase = kMode == kNTUpGate ? kt / kt_per_phase : 0;
       const int64_t k0 = static_cast<int64_t>(kt - phase * kt_per_phase) * BK;
       const uint16_t* b = reinterpret_cast<const uint16_t*>(phase == 0 ? p.b0 : p.b1) +
-                          t.bank * p.bank_stride;
+                          bank * p.bank_stride;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < C::B_CHUNKS; ++i) {
         const int c = tid + kThreads * i;
-        const int64_t n = n0 + (c >> 3);
-        const int64_t k = k0 + (c & 7) * 8;
-        rb[i] = (n < p.N && k < p.K) ? ld16(b + n * p.ldb + k) : zero4;
+        int64_t n = n0 + c / (BK / 8);
+        n = n < p.N ? n : p.N - 1;
+        const int64_t k = k0 + (c % (BK / 8)) * 8;
+        if constexpr (kTail) {
+          const bool ok = k < p.K;
+          const u32x4 v = ld16(b + n * p.ldb + (ok ? k : 0));
+          rb[i] = ok ? v : zero4;
+        } else {
+          rb[i] = ld16(b + n * p.ldb + k);
+        }
       }
     } else {
       const int64_t k0 = static_cast<int64_t>(kt) * BK;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < C::B_CHUNKS; ++i) {
         const int c = tid + kThreads * i;
-        const int64_t k = k0 + (c >> 4);
-        const int nc = c & 15;
+        const int64_t k = k0 + c / (BN / 8);
+        const int nc = c % (BN / 8);
+        const bool ok = !kTail || k < p.K;
+        const int64_t kr = ok ? k : 0;
+        u32x4 v;
         if constexpr (kMode == kNNUpGate) {
-          const uint16_t* b = reinterpret_cast<const uint16_t*>(nc < 8 ? p.b0 : p.b1) +
-                              t.bank * p.bank_stride;
-          const int64_t n = n0 + (nc & 7) * 8;
-          rb[i] = (k < p.K && n < p.N) ? ld16(b + k * p.ldb + n) : zero4;
+          constexpr int kHalf = BN / 16;  // chunks of the up half
+          const uint16_t* b = reinterpret_cast<const uint16_t*>(nc < kHalf ? p.b0 : p.b1) +
+                              bank * p.bank_stride;
+          int64_t n = n0 + (nc % kHalf) * 8;
+          n = n < p.N ? n : p.N - 8;
+          v = ld16(b + kr * p.ldb + n);
         } else if constexpr (kMode == kNNFp8W) {
-          const uint8_t* b = reinterpret_cast<const uint8_t*>(p.b0) + t.bank * p.bank_stride;
-          const int64_t n = n0 + nc * 8;
-          rb[i] = (k < p.K && n < p.N)
-                      ? fp8x8_to_bf16x8(*reinterpret_cast<const u32x2*>(b + k * p.ldb + n))
-                      : zero4;
+          const uint8_t* b = reinterpret_cast<const uint8_t*>(p.b0) + bank * p.bank_stride;
+          int64_t n = n0 + nc * 8;
+          n = n < p.N ? n : p.N - 8;
+          v = fp8x8_to_bf16x8(*reinterpret_cast<const u32x2*>(b + kr * p.ldb + n));
         } else {
-          const uint16_t* b = reinterpret_cast<const uint16_t*>(p.b0) + t.bank * p.bank_stride;
-          const int64_t n = n0 + nc * 8;
-          rb[i] = (k < p.K && n < p.N) ? ld16(b + k * p.ldb + n) : zero4;
+          const uint16_t* b = reinterpret_cast<const uint16_t*>(p.b0) + bank * p.bank_stride;
+          int64_t n = n0 + nc * 8;
+          n = n < p.N ? n : p.N - 8;
+          v = ld16(b + kr * p.ldb + n);
         }
+        rb[i] = ok ? v : zero4;
       }
+    }
+  };
+  auto load_full = [&](int kt) {  // a step known not to be the partial last one
+    load_a(kt, std::false_type{});
+    load_b(kt, std::false_type{});
+  };
+  // The partial step closes the contraction -- of each of the two phases when
+  // the contraction runs over the up and the gate half in turn.
+  auto is_tail = [&](int kt) {
+    if (!has_tail) return false;
+    if constexpr (kMode == kNTUpGate) return (kt % kt_per_phase) == kt_per_phase - 1;
+    return kt == num_kt - 1;
+  };
+  auto load_tiles = [&](int kt) {
+    if (is_tail(kt)) {
+      load_a(kt, std::true_type{});
+      load_b(kt, std::true_type{});
+    } else {
+      load_full(kt);
     }
   };
   auto store_tiles = [&](int stage) {
-    uint16_t* sa = lds + stage * 2 * TILE_ELEMS;
-    uint16_t* sb = sa + TILE_ELEMS;
+    uint16_t* sa = lds + stage * (C::A_ELEMS + C::B_ELEMS);
+    uint16_t* sb = sa + C::A_ELEMS;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < C::A_CHUNKS; ++i) {
       const int c = tid + kThreads * i;
-      *reinterpret_cast<u32x4*>(sa + (c >> 3) * KC_LD + (c & 7) * 8) = ra[i];
-      if constexpr (kBContig)
-        *reinterpret_cast<u32x4*>(sb + (c >> 3) * KC_LD + (c & 7) * 8) = rb[i];
+      if constexpr (kAContig)
+        *reinterpret_cast<u32x4*>(sa + (c / (BK / 8)) * A_LD + (c % (BK / 8)) * 8) = ra[i];
       else
-        *reinterpret_cast<u32x4*>(sb + (c >> 4) * NC_LD + (c & 15) * 8) = rb[i];
+        *reinterpret_cast<u32x4*>(sa + (c / (BM / 8)) * A_LD + (c % (BM / 8)) * 8) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < C::B_CHUNKS; ++i) {
+      const int c = tid + kThreads * i;
+      if constexpr (kBContig)
+        *reinterpret_cast<u32x4*>(sb + (c / (BK / 8)) * B_LD + (c % (BK / 8)) * 8) = rb[i];
+      else
+        *reinterpret_cast<u32x4*>(sb + (c / (BN / 8)) * B_LD + (c % (BN / 8)) * 8) = rb[i];
     }
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[C::MI][C::NJ];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < C::MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < C::NJ; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  load_a(0);
-  load_b(0);
-  store_tiles(0);
-  __syncthreads();
-
-  for (int kt = 0; kt < num_kt; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < num_kt) {
-      load_a(kt + 1);
-      load_b(kt + 1);
+  // Fragment addressing (per lane).
+  const int kc_row = lane & 31, kc_k = 8 * (lane >> 5);
+  const int tr_krow = 8 * (lane >> 5) + ((lane & 15) >> 2);
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  auto read_frags = [&](const uint16_t* sa, const uint16_t* sb, int kk, bf16x8* fa, bf16x8* fb) {
+#pragma unroll
+    for (int i = 0; i < C::MI; ++i) {
+      if constexpr (kAContig)
+        fa[i] = lds_read_kc<A_LD>(sa, C::WTM * wm + 32 * i + kc_row, 16 * kk + kc_k);
+      else
+        fa[i] = lds_read_tr<A_LD>(sa, 16 * kk + tr_krow, C::WTM * wm + 32 * i + tr_col);
     }
-    const uint16_t* sa = lds + cur * 2 * TILE_ELEMS;
-    const uint16_t* sb = sa + TILE_ELEMS;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 fa[2], fb[2];
+    for (int j = 0; j < C::NJ; ++j) {
+      if constexpr (kBContig)
+        fb[j] = lds_read_kc<B_LD>(sb, C::WTN * wn + 32 * j + kc_row, 16 * kk + kc_k);
+      else
+        fb[j] = lds_read_tr<B_LD>(sb, 16 * kk + tr_krow, C::WTN * wn + 32 * j + tr_col);
+    }
+  };
+
+  // Fragment registers persist across K steps: the first fragment of step t+1
+  // is read behind the last MFMAs of step t.
+  bf16x8 fa[2][C::MI], fb[2][C::NJ];
+  static_assert(C::KK % 2 == 0, "fragment double-buffer parity");
+  constexpr int kReads = (kAContig ? C::MI : 2 * C::MI) + (kBContig ? C::NJ : 2 * C::NJ);
+  constexpr int kWrites = C::A_CHUNKS + C::B_CHUNKS;
+  constexpr int kMfma = C::MI * C::NJ;
+  using MfmaSeq = std::make_integer_sequence<int, kMfma>;
+
+  // One K step.  kStore: the tile of step kt+1 (already in registers) goes to
+  // the idle LDS buffer.  kLoad: 0 = nothing left to fetch, 1 = fetch step kt+2
+  // (a full step), 2 = fetch step kt+2 (possibly the partial last one).
+  auto k_step = [&](int kt, auto store_tag, auto load_tag) {
+    constexpr bool kStore = decltype(store_tag)::value;
+    constexpr int kLoad = decltype(load_tag)::value;
+    const int cur = kt & 1;
+    const uint16_t* sa = lds + cur * (C::A_ELEMS + C::B_ELEMS);
+    const uint16_t* sb = sa + C::A_ELEMS;
+    const uint16_t* na = lds + (cur ^ 1) * (C::A_ELEMS + C::B_ELEMS);
+    const uint16_t* nb = na + C::A_ELEMS;
+    if constexpr (kStore) store_tiles(cur ^ 1);
+    if constexpr (kLoad == 1) load_full(kt + 2);
+    if constexpr (kLoad == 2) load_tiles(kt + 2);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        fa[i] = lds_read_kc(sa, 64 * wm + 32 * i + (lane & 31), 16 * kk + 8 * (lane >> 5));
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        if constexpr (kBContig)
-          fb[j] = lds_read_kc(sb, 64 * wn + 32 * j + (lane & 31), 16 * kk + 8 * (lane >> 5));
-        else
-          fb[j] = lds_read_tr(sb, 16 * kk + 8 * (lane >> 5) + ((lane & 15) >> 2),
-                              64 * wn + 32 * j + 16 * ((lane >> 4) & 1) + 4 * (lane & 3));
+    for (int kk = 0; kk < C::KK; ++kk) {
+      if (kk + 1 < C::KK) {
+        read_frags(sa, sb, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+      } else {
+        // Everyone has written the next buffer and read its last fragment of
+        // this one; the only barrier of the step.
+        __syncthreads();
+        if constexpr (kStore) read_frags(na, nb, 0, fa[0], fb[0]);
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < C::MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < C::NJ; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk & 1][j], fa[kk & 1][i],
+                                                               acc[i][j], 0, 0, 0);
+      if (kk == 0)
+        interleave_memory<kReads, kStore ? kWrites : 0, 0, kMfma>(MfmaSeq{});
+      else if (kk + 1 < C::KK)
+        interleave_memory<kReads, 0, 0, kMfma>(MfmaSeq{});
+      else
+        interleave_memory<kStore ? kReads : 0, 0, kLoad == 1 ? kWrites : 0, kMfma>(MfmaSeq{});
     }
-    if (kt + 1 < num_kt) store_tiles(cur ^ 1);
+  };
+
+  if (num_kt > 0) {
+    load_tiles(0);
+    store_tiles(0);
+    if (num_kt > 1) load_tiles(1);
+    __syncthreads();
+    read_frags(lds, lds + C::A_ELEMS, 0, fa[0], fb[0]);
+    using Store = std::true_type;
+    using NoStore = std::false_type;
+    int kt = 0;
+    // Steady state: the fetched step kt+2 is never a partial one (a two-phase
+    // contraction with a partial step per phase takes the checking variant).
+    if (kMode == kNTUpGate && has_tail) {
+      for (; kt + 3 < num_kt; ++kt) k_step(kt, Store{}, std::integral_constant<int, 2>{});
+    } else {
+      for (; kt + 3 < num_kt; ++kt) k_step(kt, Store{}, std::integral_constant<int, 1>{});
+    }
+    if (kt + 2 < num_kt) {
+      k_step(kt, Store{}, std::integral_constant<int, 2>{});
+      ++kt;
+    }
+    if (kt + 1 < num_kt) {
+      k_step(kt, Store{}, std::integral_constant<int, 0>{});
+      ++kt;
+    }
+    k_step(kt, NoStore{}, std::integral_constant<int, 0>{});
+  } else {
     __syncthreads();
   }
 
-  // Epilogue: bf16 tile through LDS, then coalesced 128-bit stores.
+  // ---- epilogue: bf16 tile through LDS, then coalesced 128-bit stores -----
   uint16_t* stage = lds;
-  if constexpr (kMode == kNNFp8W)
-    stage_accumulators<true>(stage, acc, wm, wn, lane, p.scale + t.bank * p.N, n0, p.N);
-  else
-    stage_accumulators<false>(stage, acc, wm, wn, lane, nullptr, 0, 0);
+  const float* col_scale = kMode == kNNFp8W ? p.scale + bank * p.N : nullptr;
+#pragma unroll
+  for (int i = 0; i < C::MI; ++i)
+#pragma unroll
+    for (int j = 0; j < C::NJ; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = C::WTM * wm + 32 * i + (lane & 31);
+        const int n = C::WTN * wn + 32 * j + 8 * q + 4 * (lane >> 5);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
+        if constexpr (kMode == kNNFp8W) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] *= (n0 + n + e < p.N) ? col_scale[n0 + n + e] : 0.0f;
+        }
+        u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        *reinterpret_cast<u32x2*>(stage + m * C::STAGE_LD + n) = packed;
+      }
   __syncthreads();
   if constexpr (kUpGateFwd) {
-    for (int c = tid; c < BM * 8; c += kThreads) {
-      const int row = c >> 3;
-      const int hc = c & 7;
+    constexpr int kHalfChunks = BN / 16;
+    for (int c = tid; c < BM * kHalfChunks; c += kThreads) {
+      const int row = c / kHalfChunks;
+      const int hc = c % kHalfChunks;
       const int64_t n = n0 + hc * 8;
-      if (row < t.nrows && n < p.N) {
-        const int64_t r = t.row0 + row;
-        const u32x4 up = *reinterpret_cast<const u32x4*>(stage + row * STAGE_LD + hc * 8);
+      if (row < nrows && n < p.N) {
+        const int64_t r = row0 + row;
+        const u32x4 up = *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + hc * 8);
         const u32x4 gate =
-            *reinterpret_cast<const u32x4*>(stage + row * STAGE_LD + 64 + hc * 8);
+            *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + BN / 2 + hc * 8);
         if (p.out != nullptr) {
           st16(p.out + r * p.ldo + n, up);
           st16(p.out + r * p.ldo + p.N + n, gate);
@@ -329,127 +537,37 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
         st16(p.out2 + r * p.ldo2 + n, pack8(h));
       }
     }
+  } else if constexpr (kMode == kTN) {
+    uint16_t* out = p.out + bank * p.bank_stride;
+    for (int c = tid; c < BM * (BN / 8); c += kThreads) {
+      const int64_t m = m0 + c / (BN / 8);
+      const int64_t n = n0 + (c % (BN / 8)) * 8;
+      if (m < p.M && n < p.N)
+        st16(out + m * p.ldo + n,
+             *reinterpret_cast<const u32x4*>(stage + (c / (BN / 8)) * C::STAGE_LD +
+                                             (c % (BN / 8)) * 8));
+    }
   } else {
-    for (int c = tid; c < BM * 16; c += kThreads) {
-      const int row = c >> 4;
-      const int64_t n = n0 + (c & 15) * 8;
-      if (row < t.nrows && n < p.N)
-        st16(p.out + (t.row0 + row) * p.ldo + n,
-             *reinterpret_cast<const u32x4*>(stage + row * STAGE_LD + (c & 15) * 8));
+    for (int c = tid; c < BM * (BN / 8); c += kThreads) {
+      const int row = c / (BN / 8);
+      const int64_t n = n0 + (c % (BN / 8)) * 8;
+      if (row < nrows && n < p.N)
+        st16(p.out + (row0 + row) * p.ldo + n,
+             *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + (c % (BN / 8)) * 8));
     }
   }
 }
 
-struct WgradParams {
-  const uint16_t* a;
-  int64_t lda;
-  const uint16_t* g;
-  int64_t ldg;
-  uint16_t* out;
-  int64_t ldo;
-  int64_t bank_stride;
-  int64_t M;
-  int64_t N;
-  int64_t rows_pad;
-  const int32_t* offs;
-  const int64_t* seg_start;
-  const int64_t* seg_count;
-};
+// Tile configurations.  Row-tiled modes need BM == NESTOR_HIP_TILE_M.
+using CfgSmall = Cfg<128, 128, 64, 2, 2>;   // wavefront tile 64 x 64
+using CfgWide = Cfg<128, 256, 64, 2, 2>;    // wavefront tile 64 x 128
+using CfgXWide = Cfg<128, 512, 32, 1, 4>;   // wavefront tile 128 x 128
+using CfgSquare = Cfg<256, 256, 64, 2, 2>;  // wavefront tile 128 x 128 (weight gradient)
+static_assert(NESTOR_HIP_TILE_M == 128, "tile table granularity");
 
-// out[e] = a[seg(e)]^T @ g[seg(e)]: both operands are contraction-major.
-__global__ __launch_bounds__(kThreads) void grouped_wgrad_kernel(WgradParams p) {
-  extern __shared__ __align__(16) uint16_t lds[];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1;
-  const int wn = wave & 1;
-  const int bank = blockIdx.z;
-  const int64_t m0 = static_cast<int64_t>(blockIdx.y) * BM;
-  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * BN;
-  int64_t seg_begin, seg_end;
-  if (p.seg_start != nullptr) {
-    seg_begin = p.seg_start[bank];
-    seg_end = seg_begin + p.seg_count[bank];
-  } else {
-    seg_begin = bank == 0 ? 0 : p.offs[bank - 1];
-    seg_end = p.offs[bank];
-  }
-  if (seg_end > p.rows_pad) seg_end = p.rows_pad;
-  const int num_kt = seg_end > seg_begin ? static_cast<int>((seg_end - seg_begin + BK - 1) / BK) : 0;
-
-  u32x4 ra[4], rb[4];
-  const u32x4 zero4 = {0, 0, 0, 0};
-  auto load_tiles = [&](int kt) {
-    const int64_t r0 = seg_begin + static_cast<int64_t>(kt) * BK;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + kThreads * i;
-      const int64_t r = r0 + (c >> 4);
-      const int cc = (c & 15) * 8;
-      ra[i] = (r < seg_end && m0 + cc < p.M) ? ld16(p.a + r * p.lda + m0 + cc) : zero4;
-      rb[i] = (r < seg_end && n0 + cc < p.N) ? ld16(p.g + r * p.ldg + n0 + cc) : zero4;
-    }
-  };
-  auto store_tiles = [&](int stage) {
-    uint16_t* sa = lds + stage * 2 * TILE_ELEMS;
-    uint16_t* sb = sa + TILE_ELEMS;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = tid + kThreads * i;
-      *reinterpret_cast<u32x4*>(sa + (c >> 4) * NC_LD + (c & 15) * 8) = ra[i];
-      *reinterpret_cast<u32x4*>(sb + (c >> 4) * NC_LD + (c & 15) * 8) = rb[i];
-    }
-  };
-
-  f32x16 acc[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-
-  if (num_kt > 0) {
-    load_tiles(0);
-    store_tiles(0);
-  }
-  __syncthreads();
-  for (int kt = 0; kt < num_kt; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < num_kt) load_tiles(kt + 1);
-    const uint16_t* sa = lds + cur * 2 * TILE_ELEMS;
-    const uint16_t* sb = sa + TILE_ELEMS;
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 fa[2], fb[2];
-      const int krow = 16 * kk + 8 * (lane >> 5) + ((lane & 15) >> 2);
-      const int cofs = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) fa[i] = lds_read_tr(sa, krow, 64 * wm + 32 * i + cofs);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) fb[j] = lds_read_tr(sb, krow, 64 * wn + 32 * j + cofs);
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < num_kt) store_tiles(cur ^ 1);
-    __syncthreads();
-  }
-
-  uint16_t* stage = lds;
-  stage_accumulators<false>(stage, acc, wm, wn, lane, nullptr, 0, 0);
-  __syncthreads();
-  uint16_t* out = p.out + bank * p.bank_stride;
-  for (int c = tid; c < BM * 16; c += kThreads) {
-    const int64_t m = m0 + (c >> 4);
-    const int64_t n = n0 + (c & 15) * 8;
-    if (m < p.M && n < p.N)
-      st16(out + m * p.ldo + n,
-           *reinterpret_cast<const u32x4*>(stage + (c >> 4) * STAGE_LD + (c & 15) * 8));
-  }
+int config_choice(const char* name, int fallback) {
+  const char* v = std::getenv(name);
+  return v != nullptr ? std::atoi(v) : fallback;
 }
 
 bool dims_ok(int64_t rows_pad, int64_t K, int64_t N, int32_t num_banks, int64_t max_tiles) {
@@ -457,19 +575,54 @@ bool dims_ok(int64_t rows_pad, int64_t K, int64_t N, int32_t num_banks, int64_t 
          N % 8 == 0 && num_banks > 0 && max_tiles > 0;
 }
 
-template <int kMode>
-int launch_gemm(const GemmParams& p, int64_t max_tiles, void* stream) {
-  const int64_t blocks = max_tiles * p.n_tiles;
+template <typename C, int kMode>
+int launch_rows(GemmParams p, void* stream) {
+  constexpr int out_cols = kMode == kNNUpGate ? C::BN / 2 : C::BN;
+  p.n_tiles = static_cast<int>(ceil_div(p.N, out_cols));
+  const int64_t blocks = p.max_tiles * p.n_tiles;
   if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_kernel<kMode>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_kernel<C, kMode>),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(kGemmLds));
+                              static_cast<int>(C::LDS_BYTES));
     configured = true;
   }
-  hipLaunchKernelGGL(grouped_gemm_kernel<kMode>, dim3(static_cast<unsigned>(blocks)),
-                     dim3(kThreads), kGemmLds, static_cast<hipStream_t>(stream), p);
+  hipLaunchKernelGGL((grouped_gemm_kernel<C, kMode>), dim3(static_cast<unsigned>(blocks)),
+                     dim3(kThreads), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
+  return launch_status();
+}
+
+template <int kMode>
+int dispatch_rows_gemm(const GemmParams& p, void* stream) {
+  static const int forced = config_choice("NESTOR_HIP_GEMM_CFG", -1);
+  int cfg = forced;
+  if (cfg < 0) cfg = p.N >= 512 ? 2 : (p.N >= 256 ? 1 : 0);
+  const int64_t width = kMode == kNNUpGate ? 2 * p.N : p.N;
+  if (cfg == 2 && width < 512) cfg = 1;
+  if (cfg == 1 && width < 256) cfg = 0;
+  switch (cfg) {
+    case 2: return launch_rows<CfgXWide, kMode>(p, stream);
+    case 1: return launch_rows<CfgWide, kMode>(p, stream);
+    default: return launch_rows<CfgSmall, kMode>(p, stream);
+  }
+}
+
+template <typename C>
+int launch_wgrad(const GemmParams& p, int32_t num_banks, void* stream) {
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_kernel<C, kTN>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(C::LDS_BYTES));
+    configured = true;
+  }
+  const int64_t my = ceil_div(p.M, C::BM);
+  if (my > 65535) return NESTOR_HIP_ERANGE;
+  hipLaunchKernelGGL((grouped_gemm_kernel<C, kTN>),
+                     dim3(static_cast<unsigned>(ceil_div(p.N, C::BN)), static_cast<unsigned>(my),
+                          static_cast<unsigned>(num_banks)),
+                     dim3(kThreads), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
   return launch_status();
 }
 
@@ -497,8 +650,7 @@ extern "C" int nestor_hip_grouped_gemm_nn(const void* a, const void* b, void* ou
   p.N = N;
   p.tile_table = tile_table;
   p.max_tiles = max_tiles;
-  p.n_tiles = static_cast<int>(ceil_div(N, BN));
-  return launch_gemm<kNN>(p, max_tiles, stream);
+  return dispatch_rows_gemm<kNN>(p, stream);
 }
 
 extern "C" int nestor_hip_grouped_gemm_upgate_swiglu(
@@ -523,8 +675,7 @@ extern "C" int nestor_hip_grouped_gemm_upgate_swiglu(
   p.N = H;
   p.tile_table = tile_table;
   p.max_tiles = max_tiles;
-  p.n_tiles = static_cast<int>(ceil_div(H, BN / 2));
-  return launch_gemm<kNNUpGate>(p, max_tiles, stream);
+  return dispatch_rows_gemm<kNNUpGate>(p, stream);
 }
 
 extern "C" int nestor_hip_grouped_gemm_nt(const void* a, const void* b, void* out,
@@ -546,8 +697,7 @@ extern "C" int nestor_hip_grouped_gemm_nt(const void* a, const void* b, void* ou
   p.N = N;
   p.tile_table = tile_table;
   p.max_tiles = max_tiles;
-  p.n_tiles = static_cast<int>(ceil_div(N, BN));
-  return launch_gemm<kNT>(p, max_tiles, stream);
+  return dispatch_rows_gemm<kNT>(p, stream);
 }
 
 extern "C" int nestor_hip_grouped_gemm_nt_upgate(
@@ -571,8 +721,7 @@ extern "C" int nestor_hip_grouped_gemm_nt_upgate(
   p.N = K;
   p.tile_table = tile_table;
   p.max_tiles = max_tiles;
-  p.n_tiles = static_cast<int>(ceil_div(K, BN));
-  return launch_gemm<kNTUpGate>(p, max_tiles, stream);
+  return dispatch_rows_gemm<kNTUpGate>(p, stream);
 }
 
 extern "C" int nestor_hip_grouped_gemm_fp8w_nn(const void* a, const void* b_q,
@@ -596,8 +745,7 @@ extern "C" int nestor_hip_grouped_gemm_fp8w_nn(const void* a, const void* b_q,
   p.N = N;
   p.tile_table = tile_table;
   p.max_tiles = max_tiles;
-  p.n_tiles = static_cast<int>(ceil_div(N, BN));
-  return launch_gemm<kNNFp8W>(p, max_tiles, stream);
+  return launch_rows<CfgSmall, kNNFp8W>(p, stream);
 }
 
 extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void* g,
@@ -613,11 +761,11 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
   if (!out || (!offs && !(seg_start && seg_count)) || (rows_pad > 0 && (!a || !g)))
     return NESTOR_HIP_EINVAL;
   if ((seg_start == nullptr) != (seg_count == nullptr)) return NESTOR_HIP_EINVAL;
-  WgradParams p = {};
+  GemmParams p = {};
   p.a = static_cast<const uint16_t*>(a);
   p.lda = lda;
-  p.g = static_cast<const uint16_t*>(g);
-  p.ldg = ldg;
+  p.b0 = g;
+  p.ldb = ldg;
   p.out = static_cast<uint16_t*>(out);
   p.ldo = ldo;
   p.bank_stride = bank_stride;
@@ -627,18 +775,11 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
   p.offs = offs;
   p.seg_start = seg_start;
   p.seg_count = seg_count;
-  static bool configured = false;
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_wgrad_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(kGemmLds));
-    configured = true;
+  static const int forced = config_choice("NESTOR_HIP_WGRAD_CFG", -1);
+  int cfg = forced >= 0 ? forced : ((M >= 256 && N >= 256) ? 3 : 0);
+  switch (cfg) {
+    case 3: return launch_wgrad<CfgSquare>(p, num_banks, stream);
+    case 1: return launch_wgrad<CfgWide>(p, num_banks, stream);
+    default: return launch_wgrad<CfgSmall>(p, num_banks, stream);
   }
-  const int64_t my = ceil_div(M, BM);
-  if (my > 65535) return NESTOR_HIP_ERANGE;
-  hipLaunchKernelGGL(grouped_wgrad_kernel,
-                     dim3(static_cast<unsigned>(ceil_div(N, BN)), static_cast<unsigned>(my),
-                          static_cast<unsigned>(num_banks)),
-                     dim3(kThreads), kGemmLds, static_cast<hipStream_t>(stream), p);
-  return launch_status();
 }
