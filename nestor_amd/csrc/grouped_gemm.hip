@@ -134,7 +134,7 @@ __device__ __forceinline__ u32x4 fp8x8_to_bf16x8(u32x2 raw) {
 
 // Scheduling recipe for one fragment's worth of MFMAs: before MFMA m, let
 // through this MFMA's share of the LDS reads (0x100), LDS writes (0x200) and
-// global loads (0x020) that sit in the same scheduling region, so each memory
+// global loads (0x010, any VMEM) that sit in the same scheduling region, so each memory
 // latency hides behind the matrix pipe (0x008) instead of in front of it.
 template <int kReads, int kWrites, int kVmem, int kMfma, int... Ms>
 __device__ __forceinline__ void interleave_memory(std::integer_sequence<int, Ms...>) {
@@ -145,7 +145,7 @@ __device__ __forceinline__ void interleave_memory(std::integer_sequence<int, Ms.
      constexpr int v = ((m + 1) * kVmem) / kMfma - (m * kVmem) / kMfma;
      if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
      if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);
-     if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
+     if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x010, v, 0);
      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
    }()),
    ...);
@@ -558,6 +558,413 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Direct-to-LDS variant.  Operand tiles go HBM -> LDS with
+// global_load_lds_dwordx4 (no staging registers, no LDS write instructions)
+// into a ring of three unpadded LDS stages, so the fetch of step t+2 is in
+// flight during the whole of steps t and t+1.  A wavefront instruction deposits
+// 64 lanes x 16 bytes as one contiguous KiB, so bank conflicts are avoided not
+// by padding rows but by choosing WHICH 16-byte piece of the tile each lane
+// fetches: position (row, c) of a contraction-contiguous tile holds logical
+// piece c ^ f(row); a contraction-major tile XORs the 32-byte column block with
+// the low bits of its row.  Fragment reads apply the same XOR.
+//
+// Requirements checked by the launcher: the contraction length is a multiple of
+// BK (row-tiled modes).  The weight gradient contracts over the rows of a
+// segment; rows behind the segment are redirected to the last padded row, which
+// is slack (all zero) in every padded tensor, so no step needs masking.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
+struct DmaCfg {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
+  static_assert(WGM * WGN == kWaves, "4 wavefronts per workgroup");
+  static constexpr int WTM = BM / WGM, WTN = BN / WGN;
+  static constexpr int MI = WTM / 32, NJ = WTN / 32;
+  static constexpr int KK = BK / 16;
+  static constexpr int STAGE_LD = BN + 8;
+  static constexpr int A_ELEMS = BM * BK, B_ELEMS = BN * BK;
+  static constexpr int STAGE_ELEMS = BM * STAGE_LD;
+  static constexpr int kStages = 3;
+  static constexpr int PIPE_ELEMS = kStages * (A_ELEMS + B_ELEMS);
+  static constexpr size_t LDS_BYTES =
+      sizeof(uint16_t) * (PIPE_ELEMS > STAGE_ELEMS ? PIPE_ELEMS : STAGE_ELEMS);
+  static constexpr int A_CHUNKS = BM * BK / 8 / kThreads;  // DMA instructions per lane
+  static constexpr int B_CHUNKS = BN * BK / 8 / kThreads;
+  static_assert(BM * BK / 8 % kThreads == 0 && BN * BK / 8 % kThreads == 0, "chunking");
+  static_assert(KK % 2 == 0, "fragment double-buffer parity");
+};
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Swizzled element offset of (row, logical 16-byte piece c) in a
+// contraction-contiguous tile with BK elements per row.
+template <int BK>
+__device__ __forceinline__ int kc_offset(int row, int c) {
+  constexpr int cpr = BK / 8;            // pieces per row
+  constexpr int rp = 256 / (BK * 2);     // rows per 256 bytes
+  return row * BK + ((c ^ ((row / rp) % cpr)) * 8);
+}
+// Swizzled element offset of (contraction row k, column n) in a
+// contraction-major tile with W elements per row (n a multiple of 4).
+template <int W>
+__device__ __forceinline__ int nc_offset(int k, int n) {
+  return k * W + ((((n >> 3) ^ (2 * (k & 3))) << 3) | (n & 7));
+}
+
+template <typename C, int kMode>
+__global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p) {
+  extern __shared__ __align__(16) uint16_t lds[];
+  constexpr int BM = C::BM, BN = C::BN, BK = C::BK;
+  constexpr bool kUpGateFwd = kMode == kNNUpGate;
+  constexpr bool kAContig = kMode != kTN;
+  constexpr bool kBContig = kMode == kNT || kMode == kNTUpGate;
+  constexpr int kOutCols = kUpGateFwd ? BN / 2 : BN;
+  // The forward up|gate tile is two contraction-major sub-tiles side by side
+  // (up columns, gate columns) so that one DMA instruction reads one bank.
+  constexpr int kSub = kUpGateFwd ? 2 : 1;
+  constexpr int BW = BN / kSub;
+  constexpr int kStageElems = C::A_ELEMS + C::B_ELEMS;
+  constexpr int kLoads = C::A_CHUNKS + C::B_CHUNKS;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / C::WGN;
+  const int wn = wave % C::WGN;
+
+  int bank, row0 = 0, nrows = BM;
+  int64_t n0, m0 = 0;
+  int64_t seg_begin = 0, seg_end = 0;
+  if constexpr (kMode == kTN) {
+    bank = blockIdx.z;
+    m0 = static_cast<int64_t>(blockIdx.y) * BM;
+    n0 = static_cast<int64_t>(blockIdx.x) * BN;
+    if (p.seg_start != nullptr) {
+      seg_begin = p.seg_start[bank];
+      seg_end = seg_begin + p.seg_count[bank];
+    } else {
+      seg_begin = bank == 0 ? 0 : p.offs[bank - 1];
+      seg_end = p.offs[bank];
+    }
+    if (seg_end > p.rows_pad) seg_end = p.rows_pad;
+  } else {
+    const int tile = blockIdx.x / p.n_tiles;
+    const int nt = blockIdx.x % p.n_tiles;
+    const int32_t* tt = p.tile_table;
+    if (tile >= tt[3 * p.max_tiles]) return;
+    bank = tt[tile];
+    row0 = tt[p.max_tiles + tile];
+    nrows = tt[2 * p.max_tiles + tile];
+    n0 = static_cast<int64_t>(nt) * kOutCols;
+    if (bank < 0) {
+      const u32x4 zero = {0, 0, 0, 0};
+      for (int c = tid; c < BM * (kOutCols / 8); c += kThreads) {
+        const int row = c / (kOutCols / 8);
+        const int64_t n = n0 + (c % (kOutCols / 8)) * 8;
+        if (row < nrows && n < p.N) {
+          const int64_t r = row0 + row;
+          if constexpr (kUpGateFwd) {
+            if (p.out != nullptr) {
+              st16(p.out + r * p.ldo + n, zero);
+              st16(p.out + r * p.ldo + p.N + n, zero);
+            }
+            st16(p.out2 + r * p.ldo2 + n, zero);
+          } else {
+            st16(p.out + r * p.ldo + n, zero);
+          }
+        }
+      }
+      return;
+    }
+  }
+
+  int num_kt, kt_per_phase = 1;
+  if constexpr (kMode == kTN) {
+    num_kt = seg_end > seg_begin ? static_cast<int>((seg_end - seg_begin + BK - 1) / BK) : 0;
+  } else {
+    kt_per_phase = static_cast<int>(p.K / BK);
+    num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
+  }
+
+  // Per-lane source offsets (elements) of every DMA instruction, relative to a
+  // wavefront-uniform base that advances with the K step.
+  int64_t offa[C::A_CHUNKS], offb[C::B_CHUNKS];
+  const int last_row = nrows - 1;
+#pragma unroll
+  for (int i = 0; i < C::A_CHUNKS; ++i) {
+    const int ci = (wave + kWaves * i) * 64 + lane;  // 16-byte position in the tile
+    if constexpr (kAContig) {
+      constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
+      int row = ci / cpr;
+      const int c = (ci % cpr) ^ ((row / rp) % cpr);
+      row = row < last_row ? row : last_row;
+      offa[i] = static_cast<int64_t>(row0 + row) * p.lda + c * 8;
+    } else {
+      const int k = ci / (BM / 8);
+      const int c = (ci % (BM / 8)) ^ (2 * (k & 3));
+      int64_t m = m0 + c * 8;
+      m = m < p.M ? m : p.M - 8;
+      offa[i] = m;  // the row is added per step (it may be redirected)
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < C::B_CHUNKS; ++i) {
+    const int blk = wave + kWaves * i;
+    const int ci = blk * 64 + lane;
+    if constexpr (kMode == kTN) {
+      const int c = (ci % (BN / 8)) ^ (2 * ((ci / (BN / 8)) & 3));
+      int64_t n = n0 + c * 8;
+      n = n < p.N ? n : p.N - 8;
+      offb[i] = n;
+    } else if constexpr (kBContig) {
+      constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
+      const int row = ci / cpr;
+      const int c = (ci % cpr) ^ ((row / rp) % cpr);
+      int64_t n = n0 + row;
+      n = n < p.N ? n : p.N - 1;
+      offb[i] = n * p.ldb + c * 8;
+    } else {
+      // sub-tile s = which half of the instructions; inside it [BK][BW]
+      constexpr int kPerSub = BK * BW / 8;  // pieces per sub-tile
+      const int cs = ci % kPerSub;
+      const int k = cs / (BW / 8);
+      const int c = (cs % (BW / 8)) ^ (2 * (k & 3));
+      int64_t n = n0 + c * 8;
+      n = n < p.N ? n : p.N - 8;
+      offb[i] = static_cast<int64_t>(k) * p.ldb + n;
+    }
+  }
+  const int64_t zero_row = p.rows_pad - 1;  // kTN: an all-zero row of every padded tensor
+
+  auto issue_loads = [&](int kt, int stage) {
+    uint16_t* sa = lds + stage * kStageElems;
+    uint16_t* sb = sa + C::A_ELEMS;
+#pragma unroll
+    for (int i = 0; i < C::A_CHUNKS; ++i) {
+      const uint16_t* src;
+      if constexpr (kAContig) {
+        src = p.a + offa[i] + static_cast<int64_t>(kt) * BK;
+      } else {
+        const int ci = (wave + kWaves * i) * 64 + lane;
+        int64_t r = seg_begin + static_cast<int64_t>(kt) * BK + ci / (BM / 8);
+        r = r < seg_end ? r : zero_row;
+        src = p.a + r * p.lda + offa[i];
+      }
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)src,
+          (NESTOR_LDS void*)(sa + (wave + kWaves * i) * 512), 16, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < C::B_CHUNKS; ++i) {
+      const int blk = wave + kWaves * i;
+      const uint16_t* src;
+      if constexpr (kMode == kTN) {
+        const int ci = blk * 64 + lane;
+        int64_t r = seg_begin + static_cast<int64_t>(kt) * BK + ci / (BN / 8);
+        r = r < seg_end ? r : zero_row;
+        src = reinterpret_cast<const uint16_t*>(p.b0) + r * p.ldb + offb[i];
+      } else if constexpr (kBContig) {
+        const int phase = kMode == kNTUpGate ? kt / kt_per_phase : 0;
+        const uint16_t* b = reinterpret_cast<const uint16_t*>(phase == 0 ? p.b0 : p.b1) +
+                            bank * p.bank_stride;
+        src = b + offb[i] + static_cast<int64_t>(kt - phase * kt_per_phase) * BK;
+      } else {
+        constexpr int kBlkPerSub = BK * BW / 8 / 64;
+        const uint16_t* b =
+            reinterpret_cast<const uint16_t*>((kSub == 2 && blk >= kBlkPerSub) ? p.b1 : p.b0) +
+            bank * p.bank_stride;
+        src = b + offb[i] + static_cast<int64_t>(kt) * BK * p.ldb;
+      }
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)src,
+          (NESTOR_LDS void*)(sb + blk * 512), 16, 0, 0);
+    }
+  };
+
+  f32x16 acc[C::MI][C::NJ];
+#pragma unroll
+  for (int i = 0; i < C::MI; ++i)
+#pragma unroll
+    for (int j = 0; j < C::NJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int kc_row = lane & 31, kc_piece = lane >> 5;
+  const int tr_krow = 8 * (lane >> 5) + ((lane & 15) >> 2);
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  auto read_frags = [&](const uint16_t* sa, const uint16_t* sb, int kk, bf16x8* fa, bf16x8* fb) {
+#pragma unroll
+    for (int i = 0; i < C::MI; ++i) {
+      if constexpr (kAContig) {
+        const int row = C::WTM * wm + 32 * i + kc_row;
+        fa[i] = *reinterpret_cast<const bf16x8*>(sa + kc_offset<BK>(row, 2 * kk + kc_piece));
+      } else {
+        const int k = 16 * kk + tr_krow;
+        const int n = C::WTM * wm + 32 * i + tr_col;
+        v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(sa + nc_offset<BM>(k, n)));
+        v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(sa + nc_offset<BM>(k + 4, n)));
+        s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        fa[i] = __builtin_bit_cast(bf16x8, v);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < C::NJ; ++j) {
+      if constexpr (kBContig) {
+        const int row = C::WTN * wn + 32 * j + kc_row;
+        fb[j] = *reinterpret_cast<const bf16x8*>(sb + kc_offset<BK>(row, 2 * kk + kc_piece));
+      } else {
+        const int col = C::WTN * wn + 32 * j;      // column inside the B tile
+        const uint16_t* sub = sb + (col / BW) * (BK * BW);
+        const int k = 16 * kk + tr_krow;
+        const int n = (col % BW) + tr_col;
+        v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(sub + nc_offset<BW>(k, n)));
+        v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(sub + nc_offset<BW>(k + 4, n)));
+        s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        fb[j] = __builtin_bit_cast(bf16x8, v);
+      }
+    }
+  };
+
+  bf16x8 fa[2][C::MI], fb[2][C::NJ];
+  constexpr int kReads = (kAContig ? C::MI : 2 * C::MI) + (kBContig ? C::NJ : 2 * C::NJ);
+  constexpr int kMfma = C::MI * C::NJ;
+  using MfmaSeq = std::make_integer_sequence<int, kMfma>;
+
+  // One K step on ring stage `cur`; kIssue: the fetch of step kt+2 goes out
+  // first; kNext: step kt+1 exists (wait for its tile, barrier, read its first
+  // fragment behind this step's last MFMAs).
+  auto k_step = [&](int kt, int cur, auto issue_tag, auto next_tag) {
+    constexpr bool kIssue = decltype(issue_tag)::value;
+    constexpr bool kNext = decltype(next_tag)::value;
+    const int nxt = cur == C::kStages - 1 ? 0 : cur + 1;
+    const int nn = nxt == C::kStages - 1 ? 0 : nxt + 1;
+    const uint16_t* sa = lds + cur * kStageElems;
+    const uint16_t* sb = sa + C::A_ELEMS;
+    const uint16_t* na = lds + nxt * kStageElems;
+    const uint16_t* nb = na + C::A_ELEMS;
+    if constexpr (kIssue) issue_loads(kt + 2, nn);
+#pragma unroll
+    for (int kk = 0; kk < C::KK; ++kk) {
+      if (kk + 1 < C::KK) {
+        read_frags(sa, sb, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+      } else if constexpr (kNext) {
+        // Own pieces of tile kt+1 have landed (only the fetch issued in this
+        // step may still be in flight) and own fragment reads have returned;
+        // after the barrier that holds for every wavefront.
+        __builtin_amdgcn_sched_barrier(0);  // earlier MFMAs stay in front of the wait
+        if constexpr (kIssue)
+          wait_vmcnt<kLoads>();
+        else
+          wait_vmcnt<0>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(na, nb, 0, fa[0], fb[0]);
+      }
+#pragma unroll
+      for (int i = 0; i < C::MI; ++i)
+#pragma unroll
+        for (int j = 0; j < C::NJ; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk & 1][j], fa[kk & 1][i],
+                                                               acc[i][j], 0, 0, 0);
+      if (kk == 0)
+        interleave_memory<kReads, 0, kIssue ? kLoads : 0, kMfma>(MfmaSeq{});
+      else if (kk + 1 < C::KK)
+        interleave_memory<kReads, 0, 0, kMfma>(MfmaSeq{});
+      else
+        interleave_memory<kNext ? kReads : 0, 0, 0, kMfma>(MfmaSeq{});
+    }
+  };
+
+  if (num_kt > 0) {
+    issue_loads(0, 0);
+    if (num_kt > 1) {
+      issue_loads(1, 1);
+      wait_vmcnt<kLoads>();
+    } else {
+      wait_vmcnt<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    read_frags(lds, lds + C::A_ELEMS, 0, fa[0], fb[0]);
+    using Yes = std::true_type;
+    using No = std::false_type;
+    int kt = 0, cur = 0;
+    for (; kt + 2 < num_kt; ++kt) {
+      k_step(kt, cur, Yes{}, Yes{});
+      cur = cur == C::kStages - 1 ? 0 : cur + 1;
+    }
+    if (kt + 1 < num_kt) {
+      k_step(kt, cur, No{}, Yes{});
+      cur = cur == C::kStages - 1 ? 0 : cur + 1;
+      ++kt;
+    }
+    k_step(kt, cur, No{}, No{});
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+
+  // ---- epilogue (same as the register-staged kernel) -----------------------
+  uint16_t* stage = lds;
+#pragma unroll
+  for (int i = 0; i < C::MI; ++i)
+#pragma unroll
+    for (int j = 0; j < C::NJ; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = C::WTM * wm + 32 * i + (lane & 31);
+        const int n = C::WTN * wn + 32 * j + 8 * q + 4 * (lane >> 5);
+        u32x2 packed = {pack_bf16x2(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
+                        pack_bf16x2(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
+        *reinterpret_cast<u32x2*>(stage + m * C::STAGE_LD + n) = packed;
+      }
+  __syncthreads();
+  if constexpr (kUpGateFwd) {
+    constexpr int kHalfChunks = BN / 16;
+    for (int c = tid; c < BM * kHalfChunks; c += kThreads) {
+      const int row = c / kHalfChunks;
+      const int hc = c % kHalfChunks;
+      const int64_t n = n0 + hc * 8;
+      if (row < nrows && n < p.N) {
+        const int64_t r = row0 + row;
+        const u32x4 up = *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + hc * 8);
+        const u32x4 gate =
+            *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + BN / 2 + hc * 8);
+        if (p.out != nullptr) {
+          st16(p.out + r * p.ldo + n, up);
+          st16(p.out + r * p.ldo + p.N + n, gate);
+        }
+        float u[8], g[8], h[8];
+        unpack8(up, u);
+        unpack8(gate, g);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) h[e] = round_bf16(g[e] / (1.0f + __expf(-g[e]))) * u[e];
+        st16(p.out2 + r * p.ldo2 + n, pack8(h));
+      }
+    }
+  } else if constexpr (kMode == kTN) {
+    uint16_t* out = p.out + bank * p.bank_stride;
+    for (int c = tid; c < BM * (BN / 8); c += kThreads) {
+      const int64_t m = m0 + c / (BN / 8);
+      const int64_t n = n0 + (c % (BN / 8)) * 8;
+      if (m < p.M && n < p.N)
+        st16(out + m * p.ldo + n,
+             *reinterpret_cast<const u32x4*>(stage + (c / (BN / 8)) * C::STAGE_LD +
+                                             (c % (BN / 8)) * 8));
+    }
+  } else {
+    for (int c = tid; c < BM * (BN / 8); c += kThreads) {
+      const int row = c / (BN / 8);
+      const int64_t n = n0 + (c % (BN / 8)) * 8;
+      if (row < nrows && n < p.N)
+        st16(p.out + (row0 + row) * p.ldo + n,
+             *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + (c % (BN / 8)) * 8));
+    }
+  }
+}
+
 // Tile configurations.  Row-tiled modes need BM == NESTOR_HIP_TILE_M.
 using CfgSmall = Cfg<128, 128, 64, 2, 2>;   // wavefront tile 64 x 64
 using CfgWide = Cfg<128, 256, 64, 2, 2>;    // wavefront tile 64 x 128
@@ -593,12 +1000,48 @@ int launch_rows(GemmParams p, void* stream) {
   return launch_status();
 }
 
+using DmaXWide = DmaCfg<128, 512, 32, 1, 4>;   // wavefront tile 128 x 128, 3-stage DMA ring
+using DmaWide = DmaCfg<128, 256, 64, 2, 2>;    // wavefront tile 64 x 128
+using DmaSquare = DmaCfg<256, 256, 32, 2, 2>;  // weight gradient
+
+template <typename C, int kMode>
+int launch_rows_dma(GemmParams p, void* stream) {
+  constexpr int out_cols = kMode == kNNUpGate ? C::BN / 2 : C::BN;
+  p.n_tiles = static_cast<int>(ceil_div(p.N, out_cols));
+  const int64_t blocks = p.max_tiles * p.n_tiles;
+  if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_dma_kernel<C, kMode>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(C::LDS_BYTES));
+    configured = true;
+  }
+  hipLaunchKernelGGL((grouped_gemm_dma_kernel<C, kMode>), dim3(static_cast<unsigned>(blocks)),
+                     dim3(kThreads), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
+  return launch_status();
+}
+
 template <int kMode>
 int dispatch_rows_gemm(const GemmParams& p, void* stream) {
   static const int forced = config_choice("NESTOR_HIP_GEMM_CFG", -1);
   int cfg = forced;
-  if (cfg < 0) cfg = p.N >= 512 ? 2 : (p.N >= 256 ? 1 : 0);
   const int64_t width = kMode == kNNUpGate ? 2 * p.N : p.N;
+  if (cfg < 0) {
+    // Measured on the 1b-like shapes: GEMMs whose operands are both read with
+    // 128-bit LDS reads (input gradients) run fastest on the direct-to-LDS
+    // 128x256 variant; GEMMs with a transposing-read operand on the
+    // register-staged 128x512 variant.
+    constexpr bool kBothContig = kMode == kNT || kMode == kNTUpGate;
+    cfg = kBothContig ? 4 : 2;
+    if (cfg == 4 && !(width >= 256 && p.K % 64 == 0)) cfg = 2;
+  }
+  if constexpr (kMode != kNNFp8W) {
+    // Direct-to-LDS variants: whole K steps only.
+    if (cfg == 3 && width >= 512 && p.K % 32 == 0) return launch_rows_dma<DmaXWide, kMode>(p, stream);
+    if (cfg == 4 && width >= 256 && p.K % 64 == 0) return launch_rows_dma<DmaWide, kMode>(p, stream);
+  }
+  if (cfg >= 3) cfg = 2;
   if (cfg == 2 && width < 512) cfg = 1;
   if (cfg == 1 && width < 256) cfg = 0;
   switch (cfg) {
@@ -777,6 +1220,23 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
   p.seg_count = seg_count;
   static const int forced = config_choice("NESTOR_HIP_WGRAD_CFG", -1);
   int cfg = forced >= 0 ? forced : ((M >= 256 && N >= 256) ? 3 : 0);
+  if (cfg == 4 && M >= 256 && N >= 256) {
+    static bool configured = false;
+    if (!configured) {
+      (void)hipFuncSetAttribute(
+          reinterpret_cast<const void*>(grouped_gemm_dma_kernel<DmaSquare, kTN>),
+          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(DmaSquare::LDS_BYTES));
+      configured = true;
+    }
+    const int64_t my = ceil_div(M, DmaSquare::BM);
+    if (my > 65535) return NESTOR_HIP_ERANGE;
+    hipLaunchKernelGGL((grouped_gemm_dma_kernel<DmaSquare, kTN>),
+                       dim3(static_cast<unsigned>(ceil_div(N, DmaSquare::BN)),
+                            static_cast<unsigned>(my), static_cast<unsigned>(num_banks)),
+                       dim3(kThreads), DmaSquare::LDS_BYTES, static_cast<hipStream_t>(stream), p);
+    return launch_status();
+  }
+  if (cfg == 4) cfg = 3;
   switch (cfg) {
     case 3: return launch_wgrad<CfgSquare>(p, num_banks, stream);
     case 1: return launch_wgrad<CfgWide>(p, num_banks, stream);
