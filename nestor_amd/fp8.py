@@ -1,0 +1,73 @@
+"""fp8 (OCP e4m3fn) weight variant of the expert bank for the inference regime.
+
+Small batches leave most experts with 0-8 rows, so a bank call is bounded by
+streaming the weights of the experts that received a row; storing them in e4m3
+halves that traffic.  Weights are quantised per output channel
+(``scale[e, n] = absmax_k |W[e, k, n]| / 448``); activations stay bf16; the MFMA
+runs in bf16 on weights widened in registers, so the only error is the weight
+rounding.  Forward only.
+"""
+
+from __future__ import annotations
+
+from typing import NamedTuple
+
+import torch
+from torch import Tensor
+
+from nestor_amd import ops
+from nestor_amd.dispatch import dispatch_plan
+from nestor_amd.expert_kernels import combine_rows, dispatch_rows, swiglu
+
+E4M3_MAX = 448.0
+
+
+class Fp8Bank(NamedTuple):
+    """Stacked SwiGLU bank in e4m3 with fp32 per-output-channel scales."""
+
+    w_up: Tensor       # [E, d, h] float8_e4m3fn
+    w_gate: Tensor
+    w_down: Tensor     # [E, h, d]
+    s_up: Tensor       # [E, h] fp32
+    s_gate: Tensor
+    s_down: Tensor     # [E, d]
+
+
+def quantize_per_channel(w: Tensor) -> tuple[Tensor, Tensor]:
+    """``[E, K, N]`` -> (e4m3 weights, ``[E, N]`` fp32 scales), absmax scaling."""
+
+    absmax = w.float().abs().amax(dim=1)
+    scale = (absmax / E4M3_MAX).clamp_min(1e-12)
+    q = (w.float() / scale.unsqueeze(1)).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    return q.contiguous(), scale.contiguous()
+
+
+def quantize_bank(w_up: Tensor, w_gate: Tensor, w_down: Tensor) -> Fp8Bank:
+    (qu, su), (qg, sg), (qd, sd) = (quantize_per_channel(t) for t in (w_up, w_gate, w_down))
+    return Fp8Bank(qu, qg, qd, su, sg, sd)
+
+
+def dequantize(q: Tensor, scale: Tensor) -> Tensor:
+    return q.float() * scale.unsqueeze(1)
+
+
+def grouped_expert_combine_fp8(
+    x: Tensor, bank: Fp8Bank, expert_ids: Tensor, weights: Tensor, group: int
+) -> Tensor:
+    """Forward of ``grouped_expert_combine`` over an e4m3 bank:
+    ``[num_tokens, slots // group, d_out]`` in ``x``'s dtype."""
+
+    num_tokens, slots = expert_ids.shape
+    assert slots % group == 0, "group must divide the slot count"
+    num_banks = bank.w_up.shape[0]
+    with torch.no_grad():
+        plan = dispatch_plan(expert_ids.reshape(-1), num_banks, slots, torch.bfloat16)
+        x_pad = dispatch_rows(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots,
+                              torch.bfloat16)
+        up = ops.grouped_gemm_fp8w_nn(x_pad, bank.w_up, bank.s_up, plan.tile_table)
+        gate = ops.grouped_gemm_fp8w_nn(x_pad, bank.w_gate, bank.s_gate, plan.tile_table)
+        hidden = swiglu(up, gate)
+        y_pad = ops.grouped_gemm_fp8w_nn(hidden, bank.w_down, bank.s_down, plan.tile_table)
+        out = combine_rows(y_pad, plan.row_dest, plan.pad_src_row, plan.pad_valid,
+                           weights.reshape(-1), group, x.dtype)
+    return out.view(num_tokens, slots // group, -1)
