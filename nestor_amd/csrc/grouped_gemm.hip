@@ -52,8 +52,8 @@ struct Cfg {
   static constexpr int KC_LD = BK + 8;       // row stride of a contraction-contiguous tile
   static constexpr int STAGE_LD = BN + 8;    // epilogue staging row stride
   // Tile sizes in elements for the two layouts of each operand.
-  static constexpr int A_KC = BM * KC_LD, A_MC = BK * (BM + 16);
-  static constexpr int B_KC = BN * KC_LD, B_NC = BK * (BN + 16);
+  static constexpr int A_KC = BM * KC_LD, A_MC = BK * (BM + 32);
+  static constexpr int B_KC = BN * KC_LD, B_NC = BK * (BN + 32);
   static constexpr int A_ELEMS = A_KC > A_MC ? A_KC : A_MC;
   static constexpr int B_ELEMS = B_KC > B_NC ? B_KC : B_NC;
   static constexpr int STAGE_ELEMS = BM * STAGE_LD;
@@ -159,11 +159,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
   constexpr bool kAContig = kMode != kTN;                         // a is [rows, K]
   constexpr bool kBContig = kMode == kNT || kMode == kNTUpGate;   // b is [N, K]
   constexpr int kOutCols = kUpGateFwd ? BN / 2 : BN;              // output columns per tile
-  constexpr int A_LD = kAContig ? C::KC_LD : BM + 16;
-  constexpr int B_LD = kBContig ? C::KC_LD : BN + 16;
+  constexpr int A_LD = kAContig ? C::KC_LD : BM + 32;
+  constexpr int B_LD = kBContig ? C::KC_LD : BN + 32;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront-uniform: keep it scalar
   const int wm = wave / C::WGN;
   const int wn = wave % C::WGN;
 
@@ -505,7 +505,15 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
         const int n = C::WTN * wn + 32 * j + 8 * q + 4 * (lane >> 5);
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (C::MI * C::NJ == 16) {
+            // 256 accumulator registers live in AGPRs; reading them where they
+            // are used keeps the compiler from hoisting every read and spilling.
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][4 * q + e]));
+          } else {
+            v[e] = acc[i][j][4 * q + e];
+          }
+        }
         if constexpr (kMode == kNNFp8W) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] *= (n0 + n + e < p.N) ? col_scale[n0 + n + e] : 0.0f;
@@ -573,25 +581,46 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
 // BK (row-tiled modes).  The weight gradient contracts over the rows of a
 // segment; rows behind the segment are redirected to the last padded row, which
 // is slack (all zero) in every padded tensor, so no step needs masking.
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int STAGES_, int OCC_ = 1>
 struct DmaCfg {
+  static constexpr int OCC = OCC_;  // workgroups resident per CU the register budget is sized for
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
-  static_assert(WGM * WGN == kWaves, "4 wavefronts per workgroup");
+  static constexpr int WAVES = WGM * WGN, THREADS = 64 * WAVES;
+  static_assert(WAVES == 4 || WAVES == 8, "one or two wavefronts per SIMD");
   static constexpr int WTM = BM / WGM, WTN = BN / WGN;
   static constexpr int MI = WTM / 32, NJ = WTN / 32;
   static constexpr int KK = BK / 16;
   static constexpr int STAGE_LD = BN + 8;
   static constexpr int A_ELEMS = BM * BK, B_ELEMS = BN * BK;
   static constexpr int STAGE_ELEMS = BM * STAGE_LD;
-  static constexpr int kStages = 3;
+  static constexpr int kStages = STAGES_;
   static constexpr int PIPE_ELEMS = kStages * (A_ELEMS + B_ELEMS);
   static constexpr size_t LDS_BYTES =
       sizeof(uint16_t) * (PIPE_ELEMS > STAGE_ELEMS ? PIPE_ELEMS : STAGE_ELEMS);
-  static constexpr int A_CHUNKS = BM * BK / 8 / kThreads;  // DMA instructions per lane
-  static constexpr int B_CHUNKS = BN * BK / 8 / kThreads;
-  static_assert(BM * BK / 8 % kThreads == 0 && BN * BK / 8 % kThreads == 0, "chunking");
+  static constexpr int A_CHUNKS = BM * BK / 8 / THREADS;  // DMA instructions per lane
+  static constexpr int B_CHUNKS = BN * BK / 8 / THREADS;
+  static_assert(BM * BK / 8 % THREADS == 0 && BN * BK / 8 % THREADS == 0, "chunking");
   static_assert(KK % 2 == 0, "fragment double-buffer parity");
+  static_assert((A_CHUNKS + B_CHUNKS) % KK == 0, "DMA instructions split evenly over the MFMA blocks");
 };
+
+// Transposing LDS read issued as inline assembly: through the builtin the
+// compiler makes every such read wait for all outstanding LDS-DMA transfers
+// (vmcnt(0)), which serialises the whole prefetch ring.  The compiler does not
+// know the instruction touches LDS, so the code that consumes the result waits
+// with an explicit lgkmcnt(0) first.
+__device__ __forceinline__ u32x2 lds_read_tr_raw(uint32_t byte_addr) {
+  u32x2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(byte_addr));
+  return v;
+}
+__device__ __forceinline__ uint32_t lds_byte_addr(const uint16_t* p) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((NESTOR_LDS const uint16_t*)p));
+}
+__device__ __forceinline__ bf16x8 join_halves(u32x2 lo, u32x2 hi) {
+  u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+  return __builtin_bit_cast(bf16x8, v);
+}
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -610,11 +639,12 @@ __device__ __forceinline__ int kc_offset(int row, int c) {
 // contraction-major tile with W elements per row (n a multiple of 4).
 template <int W>
 __device__ __forceinline__ int nc_offset(int k, int n) {
-  return k * W + ((((n >> 3) ^ (2 * (k & 3))) << 3) | (n & 7));
+  return k * W + ((((n >> 3) ^ (4 * (k & 3))) << 3) | (n & 7));
 }
 
 template <typename C, int kMode>
-__global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p) {
+__global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(GemmParams p) {
+  constexpr int kThreads = C::THREADS, kWaves = C::WAVES;
   extern __shared__ __align__(16) uint16_t lds[];
   constexpr int BM = C::BM, BN = C::BN, BK = C::BK;
   constexpr bool kUpGateFwd = kMode == kNNUpGate;
@@ -629,7 +659,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
   constexpr int kLoads = C::A_CHUNKS + C::B_CHUNKS;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront-uniform: keep it scalar
   const int wm = wave / C::WGN;
   const int wn = wave % C::WGN;
 
@@ -702,7 +732,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
       offa[i] = static_cast<int64_t>(row0 + row) * p.lda + c * 8;
     } else {
       const int k = ci / (BM / 8);
-      const int c = (ci % (BM / 8)) ^ (2 * (k & 3));
+      const int c = (ci % (BM / 8)) ^ (4 * (k & 3));
       int64_t m = m0 + c * 8;
       m = m < p.M ? m : p.M - 8;
       offa[i] = m;  // the row is added per step (it may be redirected)
@@ -713,7 +743,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
     const int blk = wave + kWaves * i;
     const int ci = blk * 64 + lane;
     if constexpr (kMode == kTN) {
-      const int c = (ci % (BN / 8)) ^ (2 * ((ci / (BN / 8)) & 3));
+      const int c = (ci % (BN / 8)) ^ (4 * ((ci / (BN / 8)) & 3));
       int64_t n = n0 + c * 8;
       n = n < p.N ? n : p.N - 8;
       offb[i] = n;
@@ -729,7 +759,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
       constexpr int kPerSub = BK * BW / 8;  // pieces per sub-tile
       const int cs = ci % kPerSub;
       const int k = cs / (BW / 8);
-      const int c = (cs % (BW / 8)) ^ (2 * (k & 3));
+      const int c = (cs % (BW / 8)) ^ (4 * (k & 3));
       int64_t n = n0 + c * 8;
       n = n < p.N ? n : p.N - 8;
       offb[i] = static_cast<int64_t>(k) * p.ldb + n;
@@ -737,11 +767,16 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
   }
   const int64_t zero_row = p.rows_pad - 1;  // kTN: an all-zero row of every padded tensor
 
-  auto issue_loads = [&](int kt, int stage) {
+  // DMA instruction q (A pieces first, then B pieces) of K step kt into ring
+  // stage `stage`.  Steps past the end re-fetch the last step: the extra tile
+  // lands in a stage nobody reads again, and every step then issues the same
+  // number of instructions, which keeps the vmcnt bookkeeping uniform.
+  auto issue_one = [&](int kt, int stage, int q) __attribute__((always_inline)) {
+    kt = kt < num_kt ? kt : num_kt - 1;
     uint16_t* sa = lds + stage * kStageElems;
     uint16_t* sb = sa + C::A_ELEMS;
-#pragma unroll
-    for (int i = 0; i < C::A_CHUNKS; ++i) {
+    if (q < C::A_CHUNKS) {
+      const int i = q;
       const uint16_t* src;
       if constexpr (kAContig) {
         src = p.a + offa[i] + static_cast<int64_t>(kt) * BK;
@@ -754,9 +789,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
       __builtin_amdgcn_global_load_lds(
           (const __attribute__((address_space(1))) void*)src,
           (NESTOR_LDS void*)(sa + (wave + kWaves * i) * 512), 16, 0, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < C::B_CHUNKS; ++i) {
+    } else {
+      const int i = q - C::A_CHUNKS;
       const int blk = wave + kWaves * i;
       const uint16_t* src;
       if constexpr (kMode == kTN) {
@@ -793,116 +827,131 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
   const int kc_row = lane & 31, kc_piece = lane >> 5;
   const int tr_krow = 8 * (lane >> 5) + ((lane & 15) >> 2);
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
-  typedef short s16x8 __attribute__((ext_vector_type(8)));
-  auto read_frags = [&](const uint16_t* sa, const uint16_t* sb, int kk, bf16x8* fa, bf16x8* fb) {
-#pragma unroll
-    for (int i = 0; i < C::MI; ++i) {
+  // Fragment read r of a fragment set into the registers of parity `par`, in
+  // the order the MFMAs consume them: B fragment 0, the A fragments, then the
+  // remaining B fragments.  Transposed fragments arrive as two raw halves.
+  bf16x8 fa[2][C::MI], fb[2][C::NJ];
+  u32x2 fa_lo[2][C::MI], fa_hi[2][C::MI], fb_lo[2][C::NJ], fb_hi[2][C::NJ];
+  auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par) __attribute__((always_inline)) {
+    if (r >= 1 && r <= C::MI) {
+      const int i = r - 1;
       if constexpr (kAContig) {
         const int row = C::WTM * wm + 32 * i + kc_row;
-        fa[i] = *reinterpret_cast<const bf16x8*>(sa + kc_offset<BK>(row, 2 * kk + kc_piece));
+        fa[par][i] = *reinterpret_cast<const bf16x8*>(sa + kc_offset<BK>(row, 2 * kk + kc_piece));
       } else {
         const int k = 16 * kk + tr_krow;
         const int n = C::WTM * wm + 32 * i + tr_col;
-        v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(sa + nc_offset<BM>(k, n)));
-        v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(sa + nc_offset<BM>(k + 4, n)));
-        s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        fa[i] = __builtin_bit_cast(bf16x8, v);
+        const uint32_t addr = lds_byte_addr(sa + nc_offset<BM>(k, n));
+        fa_lo[par][i] = lds_read_tr_raw(addr);
+        fa_hi[par][i] = lds_read_tr_raw(addr + 8 * BM);  // four contraction rows further
       }
-    }
-#pragma unroll
-    for (int j = 0; j < C::NJ; ++j) {
+    } else {
+      const int j = r == 0 ? 0 : r - C::MI;
       if constexpr (kBContig) {
         const int row = C::WTN * wn + 32 * j + kc_row;
-        fb[j] = *reinterpret_cast<const bf16x8*>(sb + kc_offset<BK>(row, 2 * kk + kc_piece));
+        fb[par][j] = *reinterpret_cast<const bf16x8*>(sb + kc_offset<BK>(row, 2 * kk + kc_piece));
       } else {
         const int col = C::WTN * wn + 32 * j;      // column inside the B tile
         const uint16_t* sub = sb + (col / BW) * (BK * BW);
         const int k = 16 * kk + tr_krow;
         const int n = (col % BW) + tr_col;
-        v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(sub + nc_offset<BW>(k, n)));
-        v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(sub + nc_offset<BW>(k + 4, n)));
-        s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        fb[j] = __builtin_bit_cast(bf16x8, v);
+        const uint32_t addr = lds_byte_addr(sub + nc_offset<BW>(k, n));
+        fb_lo[par][j] = lds_read_tr_raw(addr);
+        fb_hi[par][j] = lds_read_tr_raw(addr + 8 * BW);
       }
     }
   };
+  auto a_frag = [&](int par, int i) __attribute__((always_inline)) -> bf16x8 {
+    if constexpr (kAContig) return fa[par][i];
+    else return join_halves(fa_lo[par][i], fa_hi[par][i]);
+  };
+  auto b_frag = [&](int par, int j) __attribute__((always_inline)) -> bf16x8 {
+    if constexpr (kBContig) return fb[par][j];
+    else return join_halves(fb_lo[par][j], fb_hi[par][j]);
+  };
+  constexpr bool kRawReads = !kAContig || !kBContig;
 
-  bf16x8 fa[2][C::MI], fb[2][C::NJ];
-  constexpr int kReads = (kAContig ? C::MI : 2 * C::MI) + (kBContig ? C::NJ : 2 * C::NJ);
+  constexpr int kReads = C::MI + C::NJ;   // fragments per set
   constexpr int kMfma = C::MI * C::NJ;
-  using MfmaSeq = std::make_integer_sequence<int, kMfma>;
+  constexpr int kLoadsPerBlock = kLoads / C::KK;
+  constexpr int S = C::kStages;
 
-  // One K step on ring stage `cur`; kIssue: the fetch of step kt+2 goes out
-  // first; kNext: step kt+1 exists (wait for its tile, barrier, read its first
-  // fragment behind this step's last MFMAs).
-  auto k_step = [&](int kt, int cur, auto issue_tag, auto next_tag) {
-    constexpr bool kIssue = decltype(issue_tag)::value;
+  // One block of MFMAs on the fragment set of parity `par`, with this block's
+  // share of the memory instructions placed between them in program order:
+  // the reads of the next fragment set (into parity par ^ 1) and kLoadsPerBlock
+  // DMA instructions starting at number l0 of K step lt.  The scheduling
+  // barriers pin that order: memory instructions issued in a burst back up the
+  // address path and stall the wavefront's matrix instructions behind them.
+  auto mfma_block = [&](int par, auto reads_tag, const uint16_t* ra, const uint16_t* rb, int rkk,
+                        int lt, int ls, int l0) __attribute__((always_inline)) {
+    constexpr bool kDoReads = decltype(reads_tag)::value;
+    // The fragments this block consumes were all requested in the previous one.
+    if constexpr (kRawReads) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < kMfma; ++m) {
+      if constexpr (kDoReads) {
+#pragma unroll
+        for (int r = m * kReads / kMfma; r < (m + 1) * kReads / kMfma; ++r)
+          read_one(ra, rb, rkk, r, par ^ 1);
+      }
+#pragma unroll
+      for (int q = m * kLoadsPerBlock / kMfma; q < (m + 1) * kLoadsPerBlock / kMfma; ++q)
+        issue_one(lt, ls, l0 + q);
+      const int j = m / C::MI, i = m % C::MI;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_frag(par, j), a_frag(par, i), acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // K step kt on ring stage cur.  Ring invariant: behind the barrier of step kt
+  // every wavefront has finished reading stage cur, so step kt+S is fetched
+  // into it, one share of its DMA instructions per MFMA block: the first share
+  // behind the barrier, the others in the leading blocks of step kt+1 (where
+  // that stage is `prv`).
+  auto k_step = [&](int kt, int cur, auto next_tag) __attribute__((always_inline)) {
     constexpr bool kNext = decltype(next_tag)::value;
-    const int nxt = cur == C::kStages - 1 ? 0 : cur + 1;
-    const int nn = nxt == C::kStages - 1 ? 0 : nxt + 1;
+    const int nxt = cur == S - 1 ? 0 : cur + 1;
+    const int prv = cur == 0 ? S - 1 : cur - 1;
     const uint16_t* sa = lds + cur * kStageElems;
     const uint16_t* sb = sa + C::A_ELEMS;
     const uint16_t* na = lds + nxt * kStageElems;
     const uint16_t* nb = na + C::A_ELEMS;
-    if constexpr (kIssue) issue_loads(kt + 2, nn);
 #pragma unroll
-    for (int kk = 0; kk < C::KK; ++kk) {
-      if (kk + 1 < C::KK) {
-        read_frags(sa, sb, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
-      } else if constexpr (kNext) {
-        // Own pieces of tile kt+1 have landed (only the fetch issued in this
-        // step may still be in flight) and own fragment reads have returned;
-        // after the barrier that holds for every wavefront.
-        __builtin_amdgcn_sched_barrier(0);  // earlier MFMAs stay in front of the wait
-        if constexpr (kIssue)
-          wait_vmcnt<kLoads>();
-        else
-          wait_vmcnt<0>();
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(na, nb, 0, fa[0], fb[0]);
-      }
-#pragma unroll
-      for (int i = 0; i < C::MI; ++i)
-#pragma unroll
-        for (int j = 0; j < C::NJ; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[kk & 1][j], fa[kk & 1][i],
-                                                               acc[i][j], 0, 0, 0);
-      if (kk == 0)
-        interleave_memory<kReads, 0, kIssue ? kLoads : 0, kMfma>(MfmaSeq{});
-      else if (kk + 1 < C::KK)
-        interleave_memory<kReads, 0, 0, kMfma>(MfmaSeq{});
-      else
-        interleave_memory<kNext ? kReads : 0, 0, 0, kMfma>(MfmaSeq{});
+    for (int kk = 0; kk + 1 < C::KK; ++kk)
+      mfma_block(kk & 1, std::true_type{}, sa, sb, kk + 1, kt + S - 1, prv,
+                 (kk + 1) * kLoadsPerBlock);
+    if constexpr (kNext) {
+      // Step kt+1 has landed once only the later steps' instructions are
+      // outstanding: steps kt+2 .. kt+S-1, all issued in full by now.
+      wait_vmcnt<(S - 2) * kLoads>();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_block((C::KK - 1) & 1, std::true_type{}, na, nb, 0, kt + S, cur, 0);
+    } else {
+      mfma_block((C::KK - 1) & 1, std::false_type{}, na, nb, 0, kt + S, cur, 0);
     }
   };
 
   if (num_kt > 0) {
-    issue_loads(0, 0);
-    if (num_kt > 1) {
-      issue_loads(1, 1);
-      wait_vmcnt<kLoads>();
-    } else {
-      wait_vmcnt<0>();
-    }
+#pragma unroll
+    for (int t = 0; t < S; ++t)
+#pragma unroll
+      for (int q = 0; q < kLoads; ++q) issue_one(t, t, q);
+    wait_vmcnt<(S - 1) * kLoads>();
     __builtin_amdgcn_s_barrier();
-    read_frags(lds, lds + C::A_ELEMS, 0, fa[0], fb[0]);
-    using Yes = std::true_type;
-    using No = std::false_type;
-    int kt = 0, cur = 0;
-    for (; kt + 2 < num_kt; ++kt) {
-      k_step(kt, cur, Yes{}, Yes{});
-      cur = cur == C::kStages - 1 ? 0 : cur + 1;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < kReads; ++r) read_one(lds, lds + C::A_ELEMS, 0, r, 0);
+    int cur = 0;
+    for (int kt = 0; kt + 1 < num_kt; ++kt) {
+      k_step(kt, cur, std::true_type{});
+      cur = cur == S - 1 ? 0 : cur + 1;
     }
-    if (kt + 1 < num_kt) {
-      k_step(kt, cur, No{}, Yes{});
-      cur = cur == C::kStages - 1 ? 0 : cur + 1;
-      ++kt;
-    }
-    k_step(kt, cur, No{}, No{});
+    k_step(num_kt - 1, cur, std::false_type{});
   }
+  wait_vmcnt<0>();
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
 
@@ -916,8 +965,18 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
       for (int q = 0; q < 4; ++q) {
         const int m = C::WTM * wm + 32 * i + (lane & 31);
         const int n = C::WTN * wn + 32 * j + 8 * q + 4 * (lane >> 5);
-        u32x2 packed = {pack_bf16x2(acc[i][j][4 * q], acc[i][j][4 * q + 1]),
-                        pack_bf16x2(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3])};
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (C::MI * C::NJ == 16) {
+            // 256 accumulator registers live in AGPRs; reading them where they
+            // are used keeps the compiler from hoisting every read and spilling.
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][4 * q + e]));
+          } else {
+            v[e] = acc[i][j][4 * q + e];
+          }
+        }
+        u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         *reinterpret_cast<u32x2*>(stage + m * C::STAGE_LD + n) = packed;
       }
   __syncthreads();
@@ -965,6 +1024,342 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_dma_kernel(GemmParams p
   }
 }
 
+// ---------------------------------------------------------------------------
+// Persistent variant of the direct-to-LDS kernel for the row-tiled modes.  One
+// workgroup per CU walks a list of output tiles; the LDS ring never drains
+// between tiles, so the fetch of the next tile's first K steps overlaps the
+// last K steps and the epilogue of the current one, and the accumulators leave
+// through a per-wavefront staging area that needs no workgroup barrier.
+//
+// Work order: output tiles are numbered so that 32 consecutive numbers form a
+// 4 (row tiles) x 8 (column tiles) rectangle, and consecutive groups of 32 go
+// to consecutive XCDs (workgroup b runs on XCD b % 8): the 32 CUs of one XCD
+// work on one rectangle at a time and share its 4 activation and 8 weight
+// panels through that XCD's L2.
+template <typename C>
+struct PersLayout {
+  static constexpr int kRingElems = C::kStages * (C::A_ELEMS + C::B_ELEMS);
+  static constexpr int kEpiLd = C::WTN + 8;
+  static constexpr int kEpiElems = 32 * kEpiLd;  // one 32-row slab per wavefront
+  static constexpr size_t LDS_BYTES = sizeof(uint16_t) * (kRingElems + C::WAVES * kEpiElems);
+};
+
+template <typename C, int kMode>
+__global__ __launch_bounds__(C::THREADS, 1) void grouped_gemm_persistent_kernel(GemmParams p) {
+  static_assert(kMode == kNN || kMode == kNT || kMode == kNNUpGate || kMode == kNTUpGate, "row-tiled");
+  constexpr int kWaves = C::WAVES;
+  extern __shared__ __align__(16) uint16_t lds[];
+  constexpr int BM = C::BM, BN = C::BN, BK = C::BK, S = C::kStages;
+  constexpr bool kUpGateFwd = kMode == kNNUpGate;
+  constexpr bool kBContig = kMode == kNT || kMode == kNTUpGate;
+  constexpr int kOutCols = kUpGateFwd ? BN / 2 : BN;
+  constexpr int kSub = kUpGateFwd ? 2 : 1;
+  constexpr int BW = BN / kSub;
+  constexpr int kStageElems = C::A_ELEMS + C::B_ELEMS;
+  constexpr int kLoads = C::A_CHUNKS + C::B_CHUNKS;
+  constexpr int kLoadsPerBlock = kLoads / C::KK;
+  constexpr int kReads = C::MI + C::NJ;
+  constexpr int kMfma = C::MI * C::NJ;
+  using L = PersLayout<C>;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WGN;
+  const int wn = wave % C::WGN;
+
+  // ---- work list -----------------------------------------------------------
+  const int32_t* tt = p.tile_table;
+  const int num_rt = tt[3 * p.max_tiles + 1];  // row tiles of BM rows
+  const int n_tiles = p.n_tiles;
+  const int per_xcd = gridDim.x >> 3;
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const bool rect = per_xcd == 32 && (n_tiles & 7) == 0;
+  const int band_items = 4 * n_tiles;
+  const int w_end = rect ? ((num_rt + 3) >> 2) * band_items : num_rt * n_tiles;
+  // i-th item of this workgroup -> (row tile, column tile); false past the end.
+  auto decode = [&](int i, int& mt, int& nt) __attribute__((always_inline)) -> bool {
+    const int w = (i * 8 + xcd) * per_xcd + slot;
+    if (w >= w_end) return false;
+    if (rect) {
+      const int band = w / band_items;
+      const int r = w - band * band_items;
+      mt = band * 4 + ((r & 31) >> 3);
+      nt = (r >> 5) * 8 + (r & 7);
+    } else {
+      mt = w / n_tiles;
+      nt = w - mt * n_tiles;
+    }
+    return mt < num_rt;
+  };
+  int count = 0;
+  {
+    int mt, nt;
+    while (decode(count, mt, nt)) ++count;
+  }
+  if (count == 0) return;
+  const int kt_per_phase = static_cast<int>(p.K / BK);
+  const int num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
+
+  // ---- load cursor -----------------------------------------------------------
+  int64_t offa[C::A_CHUNKS], offb[C::B_CHUNKS];
+  int l_item = 0, l_kt = 0, l_stage = 0;
+  auto set_load_item = [&](int i) __attribute__((always_inline)) {
+    int mt, nt;
+    decode(i, mt, nt);
+    const int bank = tt[mt];
+    const int row0 = tt[p.max_tiles + mt];
+    const int nrows = tt[2 * p.max_tiles + mt];
+    const int64_t n0 = static_cast<int64_t>(nt) * kOutCols;
+    const int last_row = nrows - 1;
+#pragma unroll
+    for (int c = 0; c < C::A_CHUNKS; ++c) {
+      const int ci = (wave + kWaves * c) * 64 + lane;
+      constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
+      int row = ci / cpr;
+      const int pc = (ci % cpr) ^ ((row / rp) % cpr);
+      row = row < last_row ? row : last_row;
+      offa[c] = static_cast<int64_t>(row0 + row) * p.lda + pc * 8;
+    }
+#pragma unroll
+    for (int c = 0; c < C::B_CHUNKS; ++c) {
+      const int ci = (wave + kWaves * c) * 64 + lane;
+      if constexpr (kBContig) {
+        constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
+        const int row = ci / cpr;
+        const int pc = (ci % cpr) ^ ((row / rp) % cpr);
+        int64_t n = n0 + row;
+        n = n < p.N ? n : p.N - 1;
+        offb[c] = bank * p.bank_stride + n * p.ldb + pc * 8;
+      } else {
+        constexpr int kPerSub = BK * BW / 8;
+        const int cs = ci % kPerSub;
+        const int k = cs / (BW / 8);
+        const int pc = (cs % (BW / 8)) ^ (4 * (k & 3));
+        int64_t n = n0 + pc * 8;
+        n = n < p.N ? n : p.N - 8;
+        offb[c] = bank * p.bank_stride + static_cast<int64_t>(k) * p.ldb + n;
+      }
+    }
+  };
+  // DMA instruction q of the cursor's K step into the cursor's ring stage.
+  auto issue_one = [&](int q) __attribute__((always_inline)) {
+    uint16_t* sa = lds + l_stage * kStageElems;
+    uint16_t* sb = sa + C::A_ELEMS;
+    if (q < C::A_CHUNKS) {
+      const uint16_t* src = p.a + offa[q] + static_cast<int64_t>(l_kt) * BK;
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)src,
+          (NESTOR_LDS void*)(sa + (wave + kWaves * q) * 512), 16, 0, 0);
+    } else {
+      const int c = q - C::A_CHUNKS;
+      const int blk = wave + kWaves * c;
+      const uint16_t* src;
+      if constexpr (kBContig) {
+        const int phase = (kMode == kNTUpGate && l_kt >= kt_per_phase) ? 1 : 0;
+        src = reinterpret_cast<const uint16_t*>(phase == 0 ? p.b0 : p.b1) + offb[c] +
+              static_cast<int64_t>(l_kt - phase * kt_per_phase) * BK;
+      } else {
+        constexpr int kBlkPerSub = BK * BW / 8 / 64;
+        src = reinterpret_cast<const uint16_t*>((kSub == 2 && blk >= kBlkPerSub) ? p.b1 : p.b0) +
+              offb[c] + static_cast<int64_t>(l_kt) * BK * p.ldb;
+      }
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)src,
+          (NESTOR_LDS void*)(sb + blk * 512), 16, 0, 0);
+    }
+  };
+  // Next K step of the work list; past the end the last step is fetched again
+  // (into a stage nobody reads), which keeps the vmcnt bookkeeping uniform.
+  auto advance = [&]() __attribute__((always_inline)) {
+    l_stage = l_stage == S - 1 ? 0 : l_stage + 1;
+    if (l_kt + 1 < num_kt) {
+      ++l_kt;
+    } else if (l_item + 1 < count) {
+      ++l_item;
+      l_kt = 0;
+      set_load_item(l_item);
+    }
+  };
+
+  // ---- fragments -------------------------------------------------------------
+  f32x16 acc[C::MI][C::NJ];
+  const int kc_row = lane & 31, kc_piece = lane >> 5;
+  const int tr_krow = 8 * (lane >> 5) + ((lane & 15) >> 2);
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  // Column of B fragment j inside the B tile.  Forward up|gate: each wavefront
+  // owns the same WTN/2 output columns of the up and of the gate sub-tile, so
+  // its epilogue finds both factors of a hidden element in its own registers.
+  auto b_col = [&](int j, int& sub) __attribute__((always_inline)) -> int {
+    if constexpr (kUpGateFwd) {
+      sub = j / (C::NJ / 2);
+      return (C::WTN / 2) * wn + 32 * (j % (C::NJ / 2));
+    } else {
+      sub = 0;
+      return C::WTN * wn + 32 * j;
+    }
+  };
+  bf16x8 fa[2][C::MI], fb[2][C::NJ];
+  u32x2 fb_lo[2][C::NJ], fb_hi[2][C::NJ];  // raw halves of transposed fragments
+  auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par) __attribute__((always_inline)) {
+    if (r >= 1 && r <= C::MI) {
+      const int i = r - 1;
+      const int row = C::WTM * wm + 32 * i + kc_row;
+      fa[par][i] = *reinterpret_cast<const bf16x8*>(sa + kc_offset<BK>(row, 2 * kk + kc_piece));
+    } else {
+      const int j = r == 0 ? 0 : r - C::MI;
+      int sub;
+      const int col = b_col(j, sub);
+      if constexpr (kBContig) {
+        const int row = col + kc_row;
+        fb[par][j] = *reinterpret_cast<const bf16x8*>(sb + kc_offset<BK>(row, 2 * kk + kc_piece));
+      } else {
+        const uint16_t* base = sb + sub * (BK * BW);
+        const int k = 16 * kk + tr_krow;
+        const uint32_t addr = lds_byte_addr(base + nc_offset<BW>(k, col + tr_col));
+        fb_lo[par][j] = lds_read_tr_raw(addr);
+        fb_hi[par][j] = lds_read_tr_raw(addr + 8 * BW);  // four contraction rows further
+      }
+    }
+  };
+  auto b_frag = [&](int par, int j) __attribute__((always_inline)) -> bf16x8 {
+    if constexpr (kBContig) {
+      return fb[par][j];
+    } else {
+      u32x4 v = {fb_lo[par][j][0], fb_lo[par][j][1], fb_hi[par][j][0], fb_hi[par][j][1]};
+      return __builtin_bit_cast(bf16x8, v);
+    }
+  };
+
+  auto mfma_block = [&](int par, const uint16_t* ra, const uint16_t* rb, int rkk, int l0) __attribute__((always_inline)) {
+    if constexpr (!kBContig) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < kMfma; ++m) {
+#pragma unroll
+      for (int r = m * kReads / kMfma; r < (m + 1) * kReads / kMfma; ++r)
+        read_one(ra, rb, rkk, r, par ^ 1);
+#pragma unroll
+      for (int q = m * kLoadsPerBlock / kMfma; q < (m + 1) * kLoadsPerBlock / kMfma; ++q)
+        issue_one(l0 + q);
+      const int j = m / C::MI, i = m % C::MI;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_frag(par, j), fa[par][i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // ---- epilogue of one output tile, per wavefront -----------------------------
+  uint16_t* epi = lds + L::kRingElems + wave * L::kEpiElems;
+  auto epilogue = [&](int item) __attribute__((always_inline)) {
+    int mt, nt;
+    decode(item, mt, nt);
+    const int row0 = tt[p.max_tiles + mt];
+    const int nrows = tt[2 * p.max_tiles + mt];
+    const int64_t n0 = static_cast<int64_t>(nt) * kOutCols;
+#pragma unroll
+    for (int i = 0; i < C::MI; ++i) {
+      __builtin_amdgcn_sched_barrier(0);  // one slab's worth of registers at a time
+#pragma unroll
+      for (int j = 0; j < C::NJ; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = 32 * j + 8 * q + 4 * (lane >> 5);
+          // Read the accumulators where they are used: left to the compiler, all
+          // 256 reads move to the top of the epilogue and spill.
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][4 * q + e]));
+          u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          *reinterpret_cast<u32x2*>(epi + (lane & 31) * L::kEpiLd + n) = packed;
+        }
+      // same wavefront wrote and reads: program order is enough
+      if constexpr (kUpGateFwd) {
+        constexpr int kHalf = C::WTN / 2;          // output columns of this wavefront
+        constexpr int kCpr = kHalf / 8;            // 16-byte pieces per row
+#pragma unroll
+        for (int c = lane; c < 32 * kCpr; c += 64) {
+          const int r = c / kCpr, pc = c % kCpr;
+          const int row = C::WTM * wm + 32 * i + r;
+          const int64_t n = n0 + kHalf * wn + pc * 8;
+          const u32x4 up = *reinterpret_cast<const u32x4*>(epi + r * L::kEpiLd + pc * 8);
+          const u32x4 gate = *reinterpret_cast<const u32x4*>(epi + r * L::kEpiLd + kHalf + pc * 8);
+          if (row < nrows && n < p.N) {
+            const int64_t gr = row0 + row;
+            if (p.out != nullptr) {
+              st16(p.out + gr * p.ldo + n, up);
+              st16(p.out + gr * p.ldo + p.N + n, gate);
+            }
+            float u[8], g[8], h[8];
+            unpack8(up, u);
+            unpack8(gate, g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[e] = round_bf16(g[e] / (1.0f + __expf(-g[e]))) * u[e];
+            st16(p.out2 + gr * p.ldo2 + n, pack8(h));
+          }
+        }
+      } else {
+        constexpr int kCpr = C::WTN / 8;
+#pragma unroll
+        for (int c = lane; c < 32 * kCpr; c += 64) {
+          const int r = c / kCpr, pc = c % kCpr;
+          const int row = C::WTM * wm + 32 * i + r;
+          const int64_t n = n0 + C::WTN * wn + pc * 8;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(epi + r * L::kEpiLd + pc * 8);
+          if (row < nrows && n < p.N) st16(p.out + (row0 + row) * p.ldo + n, v);
+        }
+      }
+    }
+  };
+
+  // ---- pipeline ----------------------------------------------------------------
+  set_load_item(0);
+#pragma unroll
+  for (int t = 0; t + 1 < S; ++t) {
+#pragma unroll
+    for (int q = 0; q < kLoads; ++q) issue_one(q);
+    advance();
+  }
+#pragma unroll
+  for (int q = 0; q < kLoadsPerBlock; ++q) issue_one(q);
+  wait_vmcnt<(S - 2) * kLoads + kLoadsPerBlock>();
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int r = 0; r < kReads; ++r) read_one(lds, lds + C::A_ELEMS, 0, r, 0);
+
+  int cur = 0;
+  for (int item = 0; item < count; ++item) {
+#pragma unroll
+    for (int i = 0; i < C::MI; ++i)
+#pragma unroll
+      for (int j = 0; j < C::NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    for (int kt = 0; kt < num_kt; ++kt) {
+      const int nxt = cur == S - 1 ? 0 : cur + 1;
+      const uint16_t* sa = lds + cur * kStageElems;
+      const uint16_t* sb = sa + C::A_ELEMS;
+      const uint16_t* na = lds + nxt * kStageElems;
+      const uint16_t* nb = na + C::A_ELEMS;
+#pragma unroll
+      for (int kk = 0; kk + 1 < C::KK; ++kk)
+        mfma_block(kk & 1, sa, sb, kk + 1, (kk + 1) * kLoadsPerBlock);
+      advance();
+      // The next K step has landed once only the later steps' transfers are
+      // outstanding.
+      wait_vmcnt<(S - 2) * kLoads>();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_block((C::KK - 1) & 1, na, nb, 0, 0);
+      cur = nxt;
+    }
+    epilogue(item);
+  }
+  wait_vmcnt<0>();
+}
+
 // Tile configurations.  Row-tiled modes need BM == NESTOR_HIP_TILE_M.
 using CfgSmall = Cfg<128, 128, 64, 2, 2>;   // wavefront tile 64 x 64
 using CfgWide = Cfg<128, 256, 64, 2, 2>;    // wavefront tile 64 x 128
@@ -1000,9 +1395,11 @@ int launch_rows(GemmParams p, void* stream) {
   return launch_status();
 }
 
-using DmaXWide = DmaCfg<128, 512, 32, 1, 4>;   // wavefront tile 128 x 128, 3-stage DMA ring
-using DmaWide = DmaCfg<128, 256, 64, 2, 2>;    // wavefront tile 64 x 128
-using DmaSquare = DmaCfg<256, 256, 32, 2, 2>;  // weight gradient
+using DmaXWide = DmaCfg<128, 512, 32, 1, 4, 3>;   // wavefront tile 128 x 128, 3-stage DMA ring
+using DmaWide = DmaCfg<128, 256, 64, 2, 2, 3>;    // wavefront tile 64 x 128
+using DmaSquare = DmaCfg<256, 256, 32, 2, 2, 3>;  // weight gradient
+using DmaWide2 = DmaCfg<128, 256, 32, 2, 2, 3, 2>;  // two workgroups per CU
+using DmaSquare8 = DmaCfg<256, 256, 32, 2, 4, 4>;  // 8 wavefronts, tile 128 x 64 each
 
 template <typename C, int kMode>
 int launch_rows_dma(GemmParams p, void* stream) {
@@ -1018,7 +1415,29 @@ int launch_rows_dma(GemmParams p, void* stream) {
     configured = true;
   }
   hipLaunchKernelGGL((grouped_gemm_dma_kernel<C, kMode>), dim3(static_cast<unsigned>(blocks)),
-                     dim3(kThreads), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
+                     dim3(C::THREADS), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
+  return launch_status();
+}
+
+using PersSquare = DmaCfg<256, 256, 32, 2, 2, 3>;
+
+template <typename C, int kMode>
+int launch_rows_persistent(GemmParams p, void* stream) {
+  constexpr int out_cols = kMode == kNNUpGate ? C::BN / 2 : C::BN;
+  p.n_tiles = static_cast<int>(ceil_div(p.N, out_cols));
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+      return NESTOR_HIP_ELAUNCH;
+    num_cus = prop.multiProcessorCount / 8 * 8;
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_persistent_kernel<C, kMode>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(PersLayout<C>::LDS_BYTES));
+  }
+  hipLaunchKernelGGL((grouped_gemm_persistent_kernel<C, kMode>), dim3(static_cast<unsigned>(num_cus)),
+                     dim3(C::THREADS), PersLayout<C>::LDS_BYTES, static_cast<hipStream_t>(stream), p);
   return launch_status();
 }
 
@@ -1028,18 +1447,22 @@ int dispatch_rows_gemm(const GemmParams& p, void* stream) {
   int cfg = forced;
   const int64_t width = kMode == kNNUpGate ? 2 * p.N : p.N;
   if (cfg < 0) {
-    // Measured on the 1b-like shapes: GEMMs whose operands are both read with
-    // 128-bit LDS reads (input gradients) run fastest on the direct-to-LDS
-    // 128x256 variant; GEMMs with a transposing-read operand on the
-    // register-staged 128x512 variant.
-    constexpr bool kBothContig = kMode == kNT || kMode == kNTUpGate;
-    cfg = kBothContig ? 4 : 2;
-    if (cfg == 4 && !(width >= 256 && p.K % 64 == 0)) cfg = 2;
+    // Measured on the 1b-like shapes: the direct-to-LDS variants win in every
+    // mode; the fused up|gate input gradient prefers the 128x256x64 tile, the
+    // others the 128x512x32 one.  Shapes they do not cover (narrow outputs, a
+    // contraction that is not a multiple of the K step) take the
+    // register-staged kernel.
+    cfg = kMode == kNTUpGate ? 4 : 3;
+    if (cfg == 4 && !(width >= 256 && p.K % 64 == 0)) cfg = 3;
+    if (cfg == 3 && !(width >= 512 && p.K % 32 == 0)) cfg = 2;
   }
   if constexpr (kMode != kNNFp8W) {
     // Direct-to-LDS variants: whole K steps only.
     if (cfg == 3 && width >= 512 && p.K % 32 == 0) return launch_rows_dma<DmaXWide, kMode>(p, stream);
     if (cfg == 4 && width >= 256 && p.K % 64 == 0) return launch_rows_dma<DmaWide, kMode>(p, stream);
+    if (cfg == 5 && width >= 256 && p.K % 32 == 0) return launch_rows_dma<DmaSquare, kMode>(p, stream);
+    if (cfg == 6 && width >= 256 && p.K % 32 == 0) return launch_rows_dma<DmaSquare8, kMode>(p, stream);
+    if (cfg == 7 && width >= 256 && p.K % 32 == 0) return launch_rows_dma<DmaWide2, kMode>(p, stream);
   }
   if (cfg >= 3) cfg = 2;
   if (cfg == 2 && width < 512) cfg = 1;
@@ -1233,7 +1656,7 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
     hipLaunchKernelGGL((grouped_gemm_dma_kernel<DmaSquare, kTN>),
                        dim3(static_cast<unsigned>(ceil_div(N, DmaSquare::BN)),
                             static_cast<unsigned>(my), static_cast<unsigned>(num_banks)),
-                       dim3(kThreads), DmaSquare::LDS_BYTES, static_cast<hipStream_t>(stream), p);
+                       dim3(DmaSquare::THREADS), DmaSquare::LDS_BYTES, static_cast<hipStream_t>(stream), p);
     return launch_status();
   }
   if (cfg == 4) cfg = 3;

@@ -33,6 +33,12 @@ SHAPES = [
     (1000, 3, 20, 512, 1024, False),  # tiny config widths
     (700, 2, 16, 200, 424, True),     # production-like odd widths, empty banks
     (2048, 2, 8, 1024, 2048, False),
+    # shapes the direct-to-LDS kernels take: K loops shorter than the prefetch
+    # ring, output widths that end inside a tile
+    (500, 2, 5, 32, 512, False),
+    (500, 2, 5, 64, 520, False),
+    (700, 2, 7, 96, 1000, True),
+    (900, 1, 3, 512, 544, False),
 ]
 
 
@@ -67,6 +73,7 @@ def test_segment_mm_forward_and_grads(cuda, tokens, slots, banks, K, N, skew):
 @pytest.mark.parametrize("tokens,slots,banks,K,H,skew", [
     (300, 2, 6, 40, 24, False), (1000, 3, 20, 512, 1024, False), (700, 2, 16, 200, 424, True),
     (2048, 1, 4, 1024, 2048, False),
+    (500, 2, 5, 64, 256, False), (600, 1, 4, 96, 520, False), (900, 2, 6, 512, 576, True),
 ])
 def test_upgate_swiglu_fused_matches_unfused(cuda, tokens, slots, banks, K, H, skew):
     """The fused up|gate + SwiGLU kernel against the oracle chain with the
