@@ -604,24 +604,43 @@ struct DmaCfg {
   static_assert((A_CHUNKS + B_CHUNKS) % KK == 0, "DMA instructions split evenly over the MFMA blocks");
 };
 
-// Transposing LDS read issued as inline assembly: through the builtin the
-// compiler makes every such read wait for all outstanding LDS-DMA transfers
-// (vmcnt(0)), which serialises the whole prefetch ring.  The compiler does not
-// know the instruction touches LDS, so the code that consumes the result waits
-// with an explicit lgkmcnt(0) first.
-__device__ __forceinline__ u32x2 lds_read_tr_raw(uint32_t byte_addr) {
-  u32x2 v;
-  asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(v) : "v"(byte_addr));
-  return v;
+// One LDS-DMA instruction: 64 lanes x 16 bytes from per-lane global addresses to
+// the KiB of LDS starting at lds_addr (wavefront-uniform).  Issued as inline
+// assembly on purpose: when the compiler knows that LDS-DMA transfers are in
+// flight it makes LDS reads it cannot disambiguate from them (every transposing
+// read) wait for vmcnt(0), which drains the whole prefetch ring.  Completion is
+// tracked by hand with wait_vmcnt; LDS reads stay ordinary compiler-tracked
+// instructions.
+__device__ __forceinline__ void dma16(const void* src, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_addr), "v"(src)
+               : "memory", "m0");
 }
 __device__ __forceinline__ uint32_t lds_byte_addr(const uint16_t* p) {
   return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((NESTOR_LDS const uint16_t*)p));
 }
-__device__ __forceinline__ bf16x8 join_halves(u32x2 lo, u32x2 hi) {
-  u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+// Eight consecutive contraction indices of one output index from a swizzled
+// contraction-major tile: two transposing reads kRowElems * 4 elements apart.
+template <int kRowElems>
+__device__ __forceinline__ bf16x8 lds_read_tr_pair(const uint16_t* p0) {
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short v4s;
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(p0));
+  v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((NESTOR_LDS v4s*)(p0 + 4 * kRowElems));
+  s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   return __builtin_bit_cast(bf16x8, v);
 }
 
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{})
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -786,9 +805,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
         r = r < seg_end ? r : zero_row;
         src = p.a + r * p.lda + offa[i];
       }
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)src,
-          (NESTOR_LDS void*)(sa + (wave + kWaves * i) * 512), 16, 0, 0);
+      dma16(src, lds_byte_addr(sa + (wave + kWaves * i) * 512));
     } else {
       const int i = q - C::A_CHUNKS;
       const int blk = wave + kWaves * i;
@@ -810,9 +827,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
             bank * p.bank_stride;
         src = b + offb[i] + static_cast<int64_t>(kt) * BK * p.ldb;
       }
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)src,
-          (NESTOR_LDS void*)(sb + blk * 512), 16, 0, 0);
+      dma16(src, lds_byte_addr(sb + blk * 512));
     }
   };
 
@@ -829,9 +844,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   // Fragment read r of a fragment set into the registers of parity `par`, in
   // the order the MFMAs consume them: B fragment 0, the A fragments, then the
-  // remaining B fragments.  Transposed fragments arrive as two raw halves.
+  // remaining B fragments.
   bf16x8 fa[2][C::MI], fb[2][C::NJ];
-  u32x2 fa_lo[2][C::MI], fa_hi[2][C::MI], fb_lo[2][C::NJ], fb_hi[2][C::NJ];
   auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par) __attribute__((always_inline)) {
     if (r >= 1 && r <= C::MI) {
       const int i = r - 1;
@@ -841,9 +855,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       } else {
         const int k = 16 * kk + tr_krow;
         const int n = C::WTM * wm + 32 * i + tr_col;
-        const uint32_t addr = lds_byte_addr(sa + nc_offset<BM>(k, n));
-        fa_lo[par][i] = lds_read_tr_raw(addr);
-        fa_hi[par][i] = lds_read_tr_raw(addr + 8 * BM);  // four contraction rows further
+        fa[par][i] = lds_read_tr_pair<BM>(sa + nc_offset<BM>(k, n));
       }
     } else {
       const int j = r == 0 ? 0 : r - C::MI;
@@ -855,21 +867,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
         const uint16_t* sub = sb + (col / BW) * (BK * BW);
         const int k = 16 * kk + tr_krow;
         const int n = (col % BW) + tr_col;
-        const uint32_t addr = lds_byte_addr(sub + nc_offset<BW>(k, n));
-        fb_lo[par][j] = lds_read_tr_raw(addr);
-        fb_hi[par][j] = lds_read_tr_raw(addr + 8 * BW);
+        fb[par][j] = lds_read_tr_pair<BW>(sub + nc_offset<BW>(k, n));
       }
     }
   };
-  auto a_frag = [&](int par, int i) __attribute__((always_inline)) -> bf16x8 {
-    if constexpr (kAContig) return fa[par][i];
-    else return join_halves(fa_lo[par][i], fa_hi[par][i]);
-  };
-  auto b_frag = [&](int par, int j) __attribute__((always_inline)) -> bf16x8 {
-    if constexpr (kBContig) return fb[par][j];
-    else return join_halves(fb_lo[par][j], fb_hi[par][j]);
-  };
-  constexpr bool kRawReads = !kAContig || !kBContig;
 
   constexpr int kReads = C::MI + C::NJ;   // fragments per set
   constexpr int kMfma = C::MI * C::NJ;
@@ -885,11 +886,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   auto mfma_block = [&](int par, auto reads_tag, const uint16_t* ra, const uint16_t* rb, int rkk,
                         int lt, int ls, int l0) __attribute__((always_inline)) {
     constexpr bool kDoReads = decltype(reads_tag)::value;
-    // The fragments this block consumes were all requested in the previous one.
-    if constexpr (kRawReads) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int m = 0; m < kMfma; ++m) {
+    static_for<kMfma>([&](auto mc) __attribute__((always_inline)) {
+      constexpr int m = decltype(mc)::value;
       if constexpr (kDoReads) {
 #pragma unroll
         for (int r = m * kReads / kMfma; r < (m + 1) * kReads / kMfma; ++r)
@@ -898,10 +896,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
 #pragma unroll
       for (int q = m * kLoadsPerBlock / kMfma; q < (m + 1) * kLoadsPerBlock / kMfma; ++q)
         issue_one(lt, ls, l0 + q);
-      const int j = m / C::MI, i = m % C::MI;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_frag(par, j), a_frag(par, i), acc[i][j], 0, 0, 0);
+      constexpr int j = m / C::MI, i = m % C::MI;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[par][j], fa[par][i], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
   };
 
   // K step kt on ring stage cur.  Ring invariant: behind the barrier of step kt
@@ -1148,9 +1146,7 @@ __global__ __launch_bounds__(C::THREADS, 1) void grouped_gemm_persistent_kernel(
     uint16_t* sb = sa + C::A_ELEMS;
     if (q < C::A_CHUNKS) {
       const uint16_t* src = p.a + offa[q] + static_cast<int64_t>(l_kt) * BK;
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)src,
-          (NESTOR_LDS void*)(sa + (wave + kWaves * q) * 512), 16, 0, 0);
+      dma16(src, lds_byte_addr(sa + (wave + kWaves * q) * 512));
     } else {
       const int c = q - C::A_CHUNKS;
       const int blk = wave + kWaves * c;
@@ -1164,9 +1160,7 @@ __global__ __launch_bounds__(C::THREADS, 1) void grouped_gemm_persistent_kernel(
         src = reinterpret_cast<const uint16_t*>((kSub == 2 && blk >= kBlkPerSub) ? p.b1 : p.b0) +
               offb[c] + static_cast<int64_t>(l_kt) * BK * p.ldb;
       }
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)src,
-          (NESTOR_LDS void*)(sb + blk * 512), 16, 0, 0);
+      dma16(src, lds_byte_addr(sb + blk * 512));
     }
   };
   // Next K step of the work list; past the end the last step is fetched again
@@ -1200,7 +1194,6 @@ __global__ __launch_bounds__(C::THREADS, 1) void grouped_gemm_persistent_kernel(
     }
   };
   bf16x8 fa[2][C::MI], fb[2][C::NJ];
-  u32x2 fb_lo[2][C::NJ], fb_hi[2][C::NJ];  // raw halves of transposed fragments
   auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par) __attribute__((always_inline)) {
     if (r >= 1 && r <= C::MI) {
       const int i = r - 1;
@@ -1216,36 +1209,23 @@ __global__ __launch_bounds__(C::THREADS, 1) void grouped_gemm_persistent_kernel(
       } else {
         const uint16_t* base = sb + sub * (BK * BW);
         const int k = 16 * kk + tr_krow;
-        const uint32_t addr = lds_byte_addr(base + nc_offset<BW>(k, col + tr_col));
-        fb_lo[par][j] = lds_read_tr_raw(addr);
-        fb_hi[par][j] = lds_read_tr_raw(addr + 8 * BW);  // four contraction rows further
+        fb[par][j] = lds_read_tr_pair<BW>(base + nc_offset<BW>(k, col + tr_col));
       }
     }
   };
-  auto b_frag = [&](int par, int j) __attribute__((always_inline)) -> bf16x8 {
-    if constexpr (kBContig) {
-      return fb[par][j];
-    } else {
-      u32x4 v = {fb_lo[par][j][0], fb_lo[par][j][1], fb_hi[par][j][0], fb_hi[par][j][1]};
-      return __builtin_bit_cast(bf16x8, v);
-    }
-  };
-
   auto mfma_block = [&](int par, const uint16_t* ra, const uint16_t* rb, int rkk, int l0) __attribute__((always_inline)) {
-    if constexpr (!kBContig) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int m = 0; m < kMfma; ++m) {
+    static_for<kMfma>([&](auto mc) __attribute__((always_inline)) {
+      constexpr int m = decltype(mc)::value;
 #pragma unroll
       for (int r = m * kReads / kMfma; r < (m + 1) * kReads / kMfma; ++r)
         read_one(ra, rb, rkk, r, par ^ 1);
 #pragma unroll
       for (int q = m * kLoadsPerBlock / kMfma; q < (m + 1) * kLoadsPerBlock / kMfma; ++q)
         issue_one(l0 + q);
-      const int j = m / C::MI, i = m % C::MI;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b_frag(par, j), fa[par][i], acc[i][j], 0, 0, 0);
+      constexpr int j = m / C::MI, i = m % C::MI;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[par][j], fa[par][i], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
   };
 
   // ---- epilogue of one output tile, per wavefront -----------------------------
@@ -1360,6 +1340,330 @@ __global__ __launch_bounds__(C::THREADS, 1) void grouped_gemm_persistent_kernel(
   wait_vmcnt<0>();
 }
 
+// ---------------------------------------------------------------------------
+// Persistent weight-gradient kernel: out[bank] = a[seg]^T @ g[seg].  A bank's
+// contraction is only as long as its segment (a few hundred rows), so a
+// one-tile workgroup spends as long filling its pipeline and storing its
+// 256 x 256 result as it does multiplying.  Here one workgroup per CU walks a
+// list of output tiles with the LDS ring running across tile boundaries: the
+// first K steps of the next tile are in flight during the last K steps and the
+// epilogue of the current one.
+//
+// Both operands are contraction-major ([row, column] with the segment row as
+// the contraction index), fetched with transposing LDS reads.  Pieces of rows
+// behind the segment end are fetched from a zero constant instead, so no K
+// step needs masking and nothing is assumed about rows outside the segments.
+// Tile (bank, mt, nt) descriptors of a workgroup's list sit in LDS, filled once
+// at start.
+// Sixteen zero bytes: the DMA source of every piece that lies behind the end of
+// its segment.
+__device__ __align__(16) const uint16_t g_zero_piece[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+
+template <typename C>
+struct WgradLayout {
+  static constexpr int kMaxItems = 1024;
+  static constexpr int kRingElems = C::kStages * (C::A_ELEMS + C::B_ELEMS);
+  static constexpr int kEpiLd = C::WTN + 8;
+  static constexpr int kEpiElems = 32 * kEpiLd;  // one 32-row slab per wavefront
+  static constexpr int kTableOffset = kRingElems + C::WAVES * kEpiElems;  // in uint16 units
+  static constexpr size_t LDS_BYTES = sizeof(uint16_t) * kTableOffset + 16 * kMaxItems;
+};
+
+template <typename C>
+__global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmParams p, int num_banks) {
+  constexpr int kWaves = C::WAVES, kThreads = C::THREADS;
+  extern __shared__ __align__(16) uint16_t lds[];
+  constexpr int BM = C::BM, BN = C::BN, BK = C::BK, S = C::kStages;
+  constexpr int kStageElems = C::A_ELEMS + C::B_ELEMS;
+  constexpr int kLoads = C::A_CHUNKS + C::B_CHUNKS;
+  constexpr int kLoadsPerBlock = kLoads / C::KK;
+  constexpr int kReads = C::MI + C::NJ;
+  constexpr int kMfma = C::MI * C::NJ;
+  using L = WgradLayout<C>;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WGN;
+  const int wn = wave % C::WGN;
+
+  // ---- work list -----------------------------------------------------------
+  // Output tiles are numbered so that 32 consecutive numbers form a rectangle of
+  // 4 row tiles x 8 column tiles of one bank, and consecutive groups of 32 go to
+  // consecutive XCDs (workgroup b runs on XCD b % 8): the CUs of an XCD share
+  // the rectangle's operand panels through that XCD's L2.
+  const int m_tiles = static_cast<int>((p.M + BM - 1) / BM);
+  const int n_tiles = static_cast<int>((p.N + BN - 1) / BN);
+  const int num_rt = num_banks * m_tiles;  // row tiles over all banks
+  const int per_xcd = gridDim.x >> 3;
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const bool rect = per_xcd == 32 && (n_tiles & 7) == 0 && (m_tiles & 3) == 0;
+  const int band_items = 4 * n_tiles;
+  const int w_end = num_rt * n_tiles;
+  auto decode = [&](int i, int& rt, int& nt) __attribute__((always_inline)) -> bool {
+    const int w = (i * 8 + xcd) * per_xcd + slot;
+    if (w >= w_end) return false;
+    if (rect) {
+      const int band = w / band_items;
+      const int r = w - band * band_items;
+      rt = band * 4 + ((r & 31) >> 3);
+      nt = (r >> 5) * 8 + (r & 7);
+    } else {
+      rt = w / n_tiles;
+      nt = w - rt * n_tiles;
+    }
+    return true;
+  };
+  int4* table = reinterpret_cast<int4*>(lds + L::kTableOffset);
+  int count = 0;
+  {
+    int rt, nt;
+    while (count < L::kMaxItems && decode(count, rt, nt)) ++count;
+  }
+  for (int i = tid; i < count; i += kThreads) {
+    int rt, nt;
+    decode(i, rt, nt);
+    const int bank = rt / m_tiles;
+    int64_t beg, end;
+    if (p.seg_start != nullptr) {
+      beg = p.seg_start[bank];
+      end = beg + p.seg_count[bank];
+    } else {
+      beg = bank == 0 ? 0 : p.offs[bank - 1];
+      end = p.offs[bank];
+    }
+    if (end > p.rows_pad) end = p.rows_pad;
+    if (end < beg) end = beg;
+    table[i] = make_int4(static_cast<int>(beg), static_cast<int>(end), rt, nt);
+  }
+  __syncthreads();
+  if (count == 0) return;
+  auto steps_of = [&](int i) __attribute__((always_inline)) -> int {
+    const int4 t = table[i];
+    return (t.y - t.x + BK - 1) / BK;
+  };
+
+  // ---- load cursor -----------------------------------------------------------
+  // Each lane fetches the same pieces (contraction row krow_x[c] of the tile, a
+  // fixed group of 8 columns) in every K step, so it keeps one running source
+  // pointer per DMA instruction and adds BK rows per step.
+  const uint16_t* pa[C::A_CHUNKS];
+  const uint16_t* pb[C::B_CHUNKS];
+  // Contraction row of piece c inside the tile: krow_base(c) + lane_krow.
+  static_assert(BM / 8 == 32 && BN / 8 == 32, "one DMA instruction covers two contraction rows");
+  const int lane_krow = lane >> 5;
+  auto krow_base = [&](int c) __attribute__((always_inline)) -> int { return 2 * (wave + kWaves * c); };
+  const int64_t step_a = static_cast<int64_t>(BK) * p.lda, step_b = static_cast<int64_t>(BK) * p.ldb;
+  int l_item = -1, l_kt = 0, l_steps = 0, l_stage = 0;
+  int l_left = 0;  // segment rows from the cursor's K step on; a step with fewer than BK is a tail
+  // Moves the cursor to the first K step of the next tile that has one; false
+  // when the list is exhausted (the cursor then stays where it is).
+  auto next_load_item = [&]() __attribute__((always_inline)) -> bool {
+    int i = l_item + 1;
+    while (i < count && steps_of(i) == 0) ++i;
+    if (i >= count) return false;
+    l_item = i;
+    const int4 t = table[i];
+    const int beg = __builtin_amdgcn_readfirstlane(t.x);
+    const int end = __builtin_amdgcn_readfirstlane(t.y);
+    const int rt = __builtin_amdgcn_readfirstlane(t.z);
+    const int nt = __builtin_amdgcn_readfirstlane(t.w);
+    l_left = end - beg;
+    l_steps = (l_left + BK - 1) / BK;
+    l_kt = 0;
+    const int m0 = (rt % m_tiles) * BM;
+    const int n0 = nt * BN;
+#pragma unroll
+    for (int c = 0; c < C::A_CHUNKS; ++c) {
+      const int ci = (wave + kWaves * c) * 64 + lane;
+      const int krow = krow_base(c) + lane_krow;
+      const int pc = (ci % (BM / 8)) ^ (4 * (krow & 3));
+      int m = m0 + pc * 8;
+      m = m < p.M ? m : static_cast<int>(p.M) - 8;
+      pa[c] = p.a + (static_cast<int64_t>(beg) + krow) * p.lda + m;
+    }
+#pragma unroll
+    for (int c = 0; c < C::B_CHUNKS; ++c) {
+      const int ci = (wave + kWaves * c) * 64 + lane;
+      const int krow = krow_base(c) + lane_krow;
+      const int pc = (ci % (BN / 8)) ^ (4 * (krow & 3));
+      int n = n0 + pc * 8;
+      n = n < p.N ? n : static_cast<int>(p.N) - 8;
+      pb[c] = reinterpret_cast<const uint16_t*>(p.b0) + (static_cast<int64_t>(beg) + krow) * p.ldb + n;
+    }
+    return true;
+  };
+  // DMA instruction q of the cursor's K step.  Pieces of rows behind the segment
+  // end come from the zero constant (their running pointers may lie outside the
+  // tensors and are not used).
+  auto issue_one = [&](int q) __attribute__((always_inline)) {
+    uint16_t* sa = lds + l_stage * kStageElems;
+    uint16_t* sb = sa + C::A_ELEMS;
+    if (q < C::A_CHUNKS) {
+      const uint16_t* src = lane_krow < l_left - krow_base(q) ? pa[q] : g_zero_piece;
+      dma16(src, lds_byte_addr(sa + (wave + kWaves * q) * 512));
+    } else {
+      const int c = q - C::A_CHUNKS;
+      const uint16_t* src = lane_krow < l_left - krow_base(c) ? pb[c] : g_zero_piece;
+      dma16(src, lds_byte_addr(sb + (wave + kWaves * c) * 512));
+    }
+  };
+  // Next K step of the work list; past the end the last step is fetched again
+  // (into a stage nobody reads), which keeps the vmcnt bookkeeping uniform.
+  auto advance = [&]() __attribute__((always_inline)) {
+    l_stage = l_stage == S - 1 ? 0 : l_stage + 1;
+    if (l_kt + 1 < l_steps) {
+      ++l_kt;
+      l_left -= BK;
+#pragma unroll
+      for (int c = 0; c < C::A_CHUNKS; ++c) pa[c] += step_a;
+#pragma unroll
+      for (int c = 0; c < C::B_CHUNKS; ++c) pb[c] += step_b;
+    } else {
+      next_load_item();
+    }
+  };
+
+  // ---- fragments -------------------------------------------------------------
+  f32x16 acc[C::MI][C::NJ];
+  const int tr_krow = 8 * (lane >> 5) + ((lane & 15) >> 2);
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  bf16x8 fa[2][C::MI], fb[2][C::NJ];
+  // Element offset of each fragment's first transposing read inside a ring
+  // stage; the second K half of the stage and the upper four contraction rows of
+  // a fragment are constant offsets from it.
+  int frag_a[C::MI], frag_b[C::NJ];
+#pragma unroll
+  for (int i = 0; i < C::MI; ++i) frag_a[i] = nc_offset<BM>(tr_krow, C::WTM * wm + 32 * i + tr_col);
+#pragma unroll
+  for (int j = 0; j < C::NJ; ++j)
+    frag_b[j] = C::A_ELEMS + nc_offset<BN>(tr_krow, C::WTN * wn + 32 * j + tr_col);
+  auto read_one = [&](int stage, auto kk_tag, int r, int par) __attribute__((always_inline)) {
+    constexpr int kk = decltype(kk_tag)::value;
+    const uint16_t* base = lds + stage * kStageElems;
+    if (r >= 1 && r <= C::MI) {
+      const int i = r - 1;
+      fa[par][i] = lds_read_tr_pair<BM>(base + frag_a[i] + kk * 16 * BM);
+    } else {
+      const int j = r == 0 ? 0 : r - C::MI;
+      fb[par][j] = lds_read_tr_pair<BN>(base + frag_b[j] + kk * 16 * BN);
+    }
+  };
+  auto mfma_block = [&](int par, int rstage, auto rkk_tag, int l0) __attribute__((always_inline)) {
+    static_for<kMfma>([&](auto mc) __attribute__((always_inline)) {
+      constexpr int m = decltype(mc)::value;
+#pragma unroll
+      for (int r = m * kReads / kMfma; r < (m + 1) * kReads / kMfma; ++r)
+        read_one(rstage, rkk_tag, r, par ^ 1);
+#pragma unroll
+      for (int q = m * kLoadsPerBlock / kMfma; q < (m + 1) * kLoadsPerBlock / kMfma; ++q)
+        issue_one(l0 + q);
+      constexpr int j = m / C::MI, i = m % C::MI;
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[par][j], fa[par][i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  // ---- epilogue of one output tile, per wavefront -----------------------------
+  uint16_t* epi = lds + L::kRingElems + wave * L::kEpiElems;
+  auto epilogue = [&](int item) __attribute__((always_inline)) {
+    const int4 t = table[item];
+    const int rt = __builtin_amdgcn_readfirstlane(t.z);
+    const int nt = __builtin_amdgcn_readfirstlane(t.w);
+    const int bank = rt / m_tiles;
+    const int m0 = (rt - bank * m_tiles) * BM;
+    const int n0 = nt * BN;
+    uint16_t* out = p.out + bank * p.bank_stride;
+#pragma unroll
+    for (int i = 0; i < C::MI; ++i) {
+      __builtin_amdgcn_sched_barrier(0);  // one slab's worth of registers at a time
+#pragma unroll
+      for (int j = 0; j < C::NJ; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = 32 * j + 8 * q + 4 * (lane >> 5);
+          // Read the accumulators where they are used: left to the compiler, all
+          // 256 reads move to the top of the epilogue and spill.
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][4 * q + e]));
+          u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          *reinterpret_cast<u32x2*>(epi + (lane & 31) * L::kEpiLd + n) = packed;
+        }
+      // The same wavefront wrote and reads: program order is enough.  All reads
+      // go out before the first store so that their latencies overlap.
+      constexpr int kCpr = C::WTN / 8;
+      constexpr int kPieces = 32 * kCpr / 64;
+      u32x4 piece[kPieces];
+#pragma unroll
+      for (int t = 0; t < kPieces; ++t) {
+        const int c = lane + 64 * t;
+        piece[t] = *reinterpret_cast<const u32x4*>(epi + (c / kCpr) * L::kEpiLd + (c % kCpr) * 8);
+      }
+#pragma unroll
+      for (int t = 0; t < kPieces; ++t) {
+        const int c = lane + 64 * t;
+        const int64_t m = m0 + C::WTM * wm + 32 * i + c / kCpr;
+        const int64_t n = n0 + C::WTN * wn + (c % kCpr) * 8;
+        if (m < p.M && n < p.N) st16(out + m * p.ldo + n, piece[t]);
+      }
+    }
+  };
+  auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < C::MI; ++i)
+#pragma unroll
+      for (int j = 0; j < C::NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  };
+
+  // ---- pipeline ----------------------------------------------------------------
+  if (!next_load_item()) {
+    // every bank of this workgroup's tiles is empty: the gradients are zero
+    zero_acc();
+    for (int item = 0; item < count; ++item) epilogue(item);
+    return;
+  }
+#pragma unroll
+  for (int t = 0; t + 1 < S; ++t) {
+#pragma unroll
+    for (int q = 0; q < kLoads; ++q) issue_one(q);
+    advance();
+  }
+#pragma unroll
+  for (int q = 0; q < kLoadsPerBlock; ++q) issue_one(q);
+  wait_vmcnt<(S - 2) * kLoads + kLoadsPerBlock>();
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int r = 0; r < kReads; ++r) read_one(0, std::integral_constant<int, 0>{}, r, 0);
+
+  int cur = 0;
+  for (int item = 0; item < count; ++item) {
+    zero_acc();
+    const int num_kt = __builtin_amdgcn_readfirstlane(steps_of(item));
+    for (int kt = 0; kt < num_kt; ++kt) {
+      const int nxt = cur == S - 1 ? 0 : cur + 1;
+      using K0 = std::integral_constant<int, 0>;
+      using K1 = std::integral_constant<int, 1>;
+      mfma_block(0, cur, K1{}, kLoadsPerBlock);
+      advance();
+      // The next K step has landed once only the later steps' transfers are
+      // outstanding.
+      wait_vmcnt<(S - 2) * kLoads>();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_block(1, nxt, K0{}, 0);
+      cur = nxt;
+    }
+    epilogue(item);
+  }
+  wait_vmcnt<0>();
+}
+
 // Tile configurations.  Row-tiled modes need BM == NESTOR_HIP_TILE_M.
 using CfgSmall = Cfg<128, 128, 64, 2, 2>;   // wavefront tile 64 x 64
 using CfgWide = Cfg<128, 256, 64, 2, 2>;    // wavefront tile 64 x 128
@@ -1399,6 +1703,7 @@ using DmaXWide = DmaCfg<128, 512, 32, 1, 4, 3>;   // wavefront tile 128 x 128, 3
 using DmaWide = DmaCfg<128, 256, 64, 2, 2, 3>;    // wavefront tile 64 x 128
 using DmaSquare = DmaCfg<256, 256, 32, 2, 2, 3>;  // weight gradient
 using DmaWide2 = DmaCfg<128, 256, 32, 2, 2, 3, 2>;  // two workgroups per CU
+using WgradPers = DmaCfg<256, 256, 32, 2, 2, 3>;  // persistent weight gradient
 using DmaSquare8 = DmaCfg<256, 256, 32, 2, 4, 4>;  // 8 wavefronts, tile 128 x 64 each
 
 template <typename C, int kMode>
@@ -1642,7 +1947,29 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
   p.seg_start = seg_start;
   p.seg_count = seg_count;
   static const int forced = config_choice("NESTOR_HIP_WGRAD_CFG", -1);
-  int cfg = forced >= 0 ? forced : ((M >= 256 && N >= 256) ? 3 : 0);
+  int cfg = forced >= 0 ? forced : ((M >= 256 && N >= 256) ? 5 : 0);
+  if (cfg == 5 && M >= 256 && N >= 256 && rows_pad <= INT32_MAX) {
+    using C = WgradPers;
+    static int num_cus = 0;
+    if (num_cus == 0) {
+      int dev = 0;
+      hipDeviceProp_t prop;
+      if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+        return NESTOR_HIP_ELAUNCH;
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(wgrad_persistent_kernel<C>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(WgradLayout<C>::LDS_BYTES));
+      num_cus = prop.multiProcessorCount / 8 * 8;
+    }
+    const int64_t items = ceil_div(M, C::BM) * ceil_div(N, C::BN) * num_banks;
+    if (num_cus >= 8 && items / num_cus + 2 <= WgradLayout<C>::kMaxItems) {
+      hipLaunchKernelGGL((wgrad_persistent_kernel<C>), dim3(static_cast<unsigned>(num_cus)),
+                         dim3(C::THREADS), WgradLayout<C>::LDS_BYTES,
+                         static_cast<hipStream_t>(stream), p, num_banks);
+      return launch_status();
+    }
+  }
+  if (cfg == 5) cfg = 3;
   if (cfg == 4 && M >= 256 && N >= 256) {
     static bool configured = false;
     if (!configured) {
