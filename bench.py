@@ -26,6 +26,8 @@ sys.path.insert(0, ROOT)
 
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
+# Private-bank up|gate kernel at the mlp_1b shape: (4161600 KiB fetched + 1622016 KiB written)
+UPGATE_HBM_BYTES_PER_LAUNCH = (4161600 + 1622016) * 1024
 
 
 def _event_ms(fn, iters: int) -> float:
@@ -124,6 +126,32 @@ def kernel_breakdown(w, tensors, iters: int = 5) -> dict:
     return out
 
 
+def traffic_probe(w, tensors) -> None:
+    """A plain copy of known size (the yardstick the HBM counters are scaled by)
+    followed by the private bank's up|gate kernel on the bench's routing."""
+
+    from nestor_amd import ops
+    from nestor_amd.dispatch import dispatch_plan
+
+    dev = tensors.x.device
+    slots = w.k_columns * w.k_private
+    banks = w.columns * w.private
+    g = torch.Generator(device=dev).manual_seed(1)
+    ids = torch.randint(0, banks, (w.tokens * slots,), generator=g, device=dev)
+    plan = dispatch_plan(ids, banks, slots, torch.bfloat16)
+    x_pad = ops.dispatch_rows_fwd(tensors.x, plan.pad_token, plan.pad_valid)
+    src = torch.empty(1 << 30, dtype=torch.bfloat16, device=dev).normal_()   # 2 GiB
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    w_up, w_gate, _ = tensors.priv
+    for _ in range(2):
+        ops.upgate_swiglu_fwd(x_pad, w_up, w_gate, plan.tile_table)
+    torch.cuda.synchronize()
+    _log(f"traffic probe done: copy of {src.numel() * 2} bytes, rows_pad={plan.rows_pad}")
+
+
 def _log(msg: str) -> None:
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
@@ -208,6 +236,9 @@ def main() -> None:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="launch one 2 GiB device copy and the dominant kernel twice, then exit: the "
+                         "command to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the expert MLP: run it with --gpus 1 "
@@ -223,6 +254,9 @@ def main() -> None:
     w = WORKLOADS[args.workload]
     dev = torch.device("cuda:0")
     tensors = make_tensors(w, args.seed, dev)
+    if args.traffic_probe:
+        traffic_probe(w, tensors)
+        return
     column_router, pool = build_pool(w, tensors)
     params = list(column_router.parameters()) + list(pool.parameters())
     x = tensors.x.clone().requires_grad_(True)
@@ -264,7 +298,10 @@ def main() -> None:
             "peak": BF16_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": dom["frac_mfma_peak"],
-            "traffic": None,
+            # HBM bytes per launch of this kernel: FETCH_SIZE + WRITE_SIZE from two
+            # `rocprofv3 --pmc` runs of `bench.py --traffic-probe`, each scaled by the
+            # same counter's reading for a device copy of known size (both factors 1.00).
+            "traffic": UPGATE_HBM_BYTES_PER_LAUNCH if w.name == "mlp_1b" else None,
         }
     result = {
         "metric": "expert-MLP fwd+bwd tokens/s @1b shape, 1 GPU; % bf16 MFMA / HBM peak",
