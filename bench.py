@@ -80,8 +80,8 @@ def kernel_breakdown(w, tensors, iters: int = 5) -> dict:
     report("index_build", ms, bytes_=rows * 8 + rows * 8 + 3 * rows_pad * 8 + rows_pad * 2 + banks * 20)
 
     x = tensors.x
-    x_pad = ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid)
-    ms = _event_ms(lambda: ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid), iters)
+    x_pad = ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots)
+    ms = _event_ms(lambda: ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots), iters)
     report("dispatch_fwd", ms, bytes_=T * d * 2 + rows * d * 2 + rows * 8)
 
     up_gate, hidden = ops.upgate_swiglu_fwd(x_pad, w_up, w_gate, plan.tile_table)

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 1
+#define NESTOR_HIP_ABI_VERSION 2
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -113,11 +113,15 @@ int nestor_hip_tile_schedule(
 
 /* x_pad[p,:] = pad_valid[p] ? bf16(x[pad_token[p],:]) : 0
  * (nestor/backbones/triton_expert.py:509-539 dispatch_rows; kernel
- * nestor/backbones/triton_packed.py:113-139).  dim % 8 == 0. */
+ * nestor/backbones/triton_packed.py:113-139).  dim % 8 == 0.
+ * row_dest (nullable, [num_tokens*slots], the inverse map dispatch_rows also
+ * receives) selects the source-major kernel for bf16 x: every token is read once
+ * and written to the rows of its assignments; same result. */
 int nestor_hip_dispatch_rows_fwd(
     const void* x, int32_t x_dtype, const int64_t* pad_token,
     const void* pad_valid, int32_t valid_dtype,
     void* x_pad /* bf16 [rows_pad, dim] */, int64_t rows_pad, int64_t dim,
+    const int64_t* row_dest, int64_t num_tokens, int32_t slots,
     void* stream);
 
 /* grad_x[t,:] = sum_{j<slots} grad_pad[row_dest[t*slots+j],:], fp32 sum,

@@ -846,8 +846,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   // the order the MFMAs consume them: B fragment 0, the A fragments, then the
   // remaining B fragments.
   bf16x8 fa[2][C::MI], fb[2][C::NJ];
-  auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par) __attribute__((always_inline)) {
-    if (r >= 1 && r <= C::MI) {
+  auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par, int mi_eff) __attribute__((always_inline)) {
+    if (r >= 1 && r <= mi_eff) {
       const int i = r - 1;
       if constexpr (kAContig) {
         const int row = C::WTM * wm + 32 * i + kc_row;
@@ -858,7 +858,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
         fa[par][i] = lds_read_tr_pair<BM>(sa + nc_offset<BM>(k, n));
       }
     } else {
-      const int j = r == 0 ? 0 : r - C::MI;
+      const int j = r == 0 ? 0 : r - mi_eff;
       if constexpr (kBContig) {
         const int row = C::WTN * wn + 32 * j + kc_row;
         fb[par][j] = *reinterpret_cast<const bf16x8*>(sb + kc_offset<BK>(row, 2 * kk + kc_piece));
@@ -883,20 +883,26 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   // DMA instructions starting at number l0 of K step lt.  The scheduling
   // barriers pin that order: memory instructions issued in a burst back up the
   // address path and stall the wavefront's matrix instructions behind them.
-  auto mfma_block = [&](int par, auto reads_tag, const uint16_t* ra, const uint16_t* rb, int rkk,
-                        int lt, int ls, int l0) __attribute__((always_inline)) {
+  // mi_tag: how many of the wavefront's 32-row blocks hold rows of the tile; the
+  // MFMAs and A fragments of the others are skipped (a segment's last tile is on
+  // average half empty, and with one row of wavefronts per tile every
+  // wavefront skips the same blocks).
+  auto mfma_block = [&](auto mi_tag, int par, auto reads_tag, const uint16_t* ra, const uint16_t* rb,
+                        int rkk, int lt, int ls, int l0) __attribute__((always_inline)) {
+    constexpr int kMi = decltype(mi_tag)::value;
     constexpr bool kDoReads = decltype(reads_tag)::value;
-    static_for<kMfma>([&](auto mc) __attribute__((always_inline)) {
+    constexpr int kMfmaEff = kMi * C::NJ, kReadsEff = kMi + C::NJ;
+    static_for<kMfmaEff>([&](auto mc) __attribute__((always_inline)) {
       constexpr int m = decltype(mc)::value;
       if constexpr (kDoReads) {
 #pragma unroll
-        for (int r = m * kReads / kMfma; r < (m + 1) * kReads / kMfma; ++r)
-          read_one(ra, rb, rkk, r, par ^ 1);
+        for (int r = m * kReadsEff / kMfmaEff; r < (m + 1) * kReadsEff / kMfmaEff; ++r)
+          read_one(ra, rb, rkk, r, par ^ 1, kMi);
       }
 #pragma unroll
-      for (int q = m * kLoadsPerBlock / kMfma; q < (m + 1) * kLoadsPerBlock / kMfma; ++q)
+      for (int q = m * kLoadsPerBlock / kMfmaEff; q < (m + 1) * kLoadsPerBlock / kMfmaEff; ++q)
         issue_one(lt, ls, l0 + q);
-      constexpr int j = m / C::MI, i = m % C::MI;
+      constexpr int j = m / kMi, i = m % kMi;
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[par][j], fa[par][i], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -907,7 +913,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   // into it, one share of its DMA instructions per MFMA block: the first share
   // behind the barrier, the others in the leading blocks of step kt+1 (where
   // that stage is `prv`).
-  auto k_step = [&](int kt, int cur, auto next_tag) __attribute__((always_inline)) {
+  auto k_step = [&](auto mi_tag, int kt, int cur, auto next_tag) __attribute__((always_inline)) {
     constexpr bool kNext = decltype(next_tag)::value;
     const int nxt = cur == S - 1 ? 0 : cur + 1;
     const int prv = cur == 0 ? S - 1 : cur - 1;
@@ -917,7 +923,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     const uint16_t* nb = na + C::A_ELEMS;
 #pragma unroll
     for (int kk = 0; kk + 1 < C::KK; ++kk)
-      mfma_block(kk & 1, std::true_type{}, sa, sb, kk + 1, kt + S - 1, prv,
+      mfma_block(mi_tag, kk & 1, std::true_type{}, sa, sb, kk + 1, kt + S - 1, prv,
                  (kk + 1) * kLoadsPerBlock);
     if constexpr (kNext) {
       // Step kt+1 has landed once only the later steps' instructions are
@@ -926,10 +932,22 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      mfma_block((C::KK - 1) & 1, std::true_type{}, na, nb, 0, kt + S, cur, 0);
+      mfma_block(mi_tag, (C::KK - 1) & 1, std::true_type{}, na, nb, 0, kt + S, cur, 0);
     } else {
-      mfma_block((C::KK - 1) & 1, std::false_type{}, na, nb, 0, kt + S, cur, 0);
+      mfma_block(mi_tag, (C::KK - 1) & 1, std::false_type{}, na, nb, 0, kt + S, cur, 0);
     }
+  };
+
+  auto k_loop = [&](auto mi_tag) __attribute__((always_inline)) {
+    constexpr int kMi = decltype(mi_tag)::value;
+#pragma unroll
+    for (int r = 0; r < kMi + C::NJ; ++r) read_one(lds, lds + C::A_ELEMS, 0, r, 0, kMi);
+    int cur = 0;
+    for (int kt = 0; kt + 1 < num_kt; ++kt) {
+      k_step(mi_tag, kt, cur, std::true_type{});
+      cur = cur == S - 1 ? 0 : cur + 1;
+    }
+    k_step(mi_tag, num_kt - 1, cur, std::false_type{});
   };
 
   if (num_kt > 0) {
@@ -940,14 +958,22 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     wait_vmcnt<(S - 1) * kLoads>();
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int r = 0; r < kReads; ++r) read_one(lds, lds + C::A_ELEMS, 0, r, 0);
-    int cur = 0;
-    for (int kt = 0; kt + 1 < num_kt; ++kt) {
-      k_step(kt, cur, std::true_type{});
-      cur = cur == S - 1 ? 0 : cur + 1;
+    // Row blocks in use: only tiles with a single row of wavefronts can skip.
+    int mi_eff = C::MI;
+    if constexpr (C::WGM == 1 && kMode != kTN && C::MI == 4) {
+      mi_eff = (nrows + 31) >> 5;
+      mi_eff = mi_eff < 1 ? 1 : (mi_eff > 4 ? 4 : mi_eff);
     }
-    k_step(num_kt - 1, cur, std::false_type{});
+    if constexpr (C::WGM == 1 && kMode != kTN && C::MI == 4) {
+      switch (mi_eff) {
+        case 1: k_loop(std::integral_constant<int, 1>{}); break;
+        case 2: k_loop(std::integral_constant<int, 2>{}); break;
+        case 3: k_loop(std::integral_constant<int, 3>{}); break;
+        default: k_loop(std::integral_constant<int, 4>{}); break;
+      }
+    } else {
+      k_loop(std::integral_constant<int, C::MI>{});
+    }
   }
   wait_vmcnt<0>();
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");

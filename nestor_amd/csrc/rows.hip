@@ -12,35 +12,68 @@ namespace {
 
 constexpr int kRowBlock = 256;
 constexpr int kRowsPerBlock = kRowBlock / kWave;
+// Pieces a lane requests before it consumes the first one.  With one piece in
+// flight per lane the kernels are bound by memory latency times occupancy
+// (about half of the HBM peak); batching the loads puts enough bytes in flight.
+constexpr int kBatch = 4;
 
 __device__ __forceinline__ int64_t wave_row() {
   return static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + threadIdx.x / kWave;
 }
 
 // x_pad[p,:] = valid[p] ? bf16(x[pad_token[p],:]) : 0
+// A wavefront moves kGatherRows consecutive padded rows: their map entries are
+// fetched together (one memory latency instead of one per row) and the pieces
+// of all of them are requested before the first store.
+constexpr int kGatherRows = 2;
 template <bool kXF32>
 __global__ __launch_bounds__(kRowBlock) void dispatch_fwd_kernel(
     const void* __restrict__ x, const int64_t* __restrict__ pad_token,
     const void* __restrict__ pad_valid, int valid_dtype, uint16_t* __restrict__ out,
     int64_t rows_pad, int64_t dim) {
-  const int64_t p = wave_row();
-  if (p >= rows_pad) return;
+  const int64_t p0 = wave_row() * kGatherRows;
+  if (p0 >= rows_pad) return;
   const int lane = threadIdx.x % kWave;
   const int chunks = static_cast<int>(dim / 8);
-  uint16_t* dst = out + p * dim;
-  if (!load_valid(pad_valid, p, valid_dtype)) {
-    const u32x4 zero = {0, 0, 0, 0};
-    for (int c = lane; c < chunks; c += kWave) st16(dst + c * 8, zero);
-    return;
+  bool valid[kGatherRows];
+  int64_t tok[kGatherRows];
+#pragma unroll
+  for (int r = 0; r < kGatherRows; ++r) {
+    const int64_t p = p0 + r < rows_pad ? p0 + r : rows_pad - 1;
+    valid[r] = load_valid(pad_valid, p, valid_dtype);
+    tok[r] = pad_token[p];  // slack entries hold 0: always a readable row
   }
-  const int64_t tok = pad_token[p];
-  for (int c = lane; c < chunks; c += kWave) {
-    if constexpr (kXF32) {
-      float f[8];
-      load8_as_f32<true>(x, tok * dim + c * 8, f);
-      st16(dst + c * 8, pack8(f));
-    } else {
-      st16(dst + c * 8, ld16(reinterpret_cast<const uint16_t*>(x) + tok * dim + c * 8));
+  if constexpr (kXF32) {
+#pragma unroll
+    for (int r = 0; r < kGatherRows; ++r) {
+      if (p0 + r >= rows_pad) break;
+      uint16_t* dst = out + (p0 + r) * dim;
+      for (int c = lane; c < chunks; c += kWave) {
+        float f[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (valid[r]) load8_as_f32<true>(x, tok[r] * dim + c * 8, f);
+        st16(dst + c * 8, pack8(f));
+      }
+    }
+  } else {
+    const u32x4 zero = {0, 0, 0, 0};
+    for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+      u32x4 v[kGatherRows][kBatch];
+#pragma unroll
+      for (int r = 0; r < kGatherRows; ++r) {
+        const uint16_t* src = reinterpret_cast<const uint16_t*>(x) + tok[r] * dim;
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b)
+          v[r][b] = (valid[r] && c0 + b * kWave < chunks) ? ld16(src + (c0 + b * kWave) * 8) : zero;
+      }
+#pragma unroll
+      for (int r = 0; r < kGatherRows; ++r) {
+        if (p0 + r < rows_pad) {
+          uint16_t* dst = out + (p0 + r) * dim;
+#pragma unroll
+          for (int b = 0; b < kBatch; ++b)
+            if (c0 + b * kWave < chunks) st16(dst + (c0 + b * kWave) * 8, v[r][b]);
+        }
+      }
     }
   }
 }
@@ -54,16 +87,31 @@ __global__ __launch_bounds__(kRowBlock) void dispatch_bwd_kernel(
   if (t >= num_tokens) return;
   const int lane = threadIdx.x % kWave;
   const int chunks = static_cast<int>(dim / 8);
-  for (int c = lane; c < chunks; c += kWave) {
-    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int j = 0; j < slots; ++j) {
-      const int64_t r = row_dest[t * slots + j];
-      float f[8];
-      unpack8(ld16(g + r * dim + c * 8), f);
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    float acc[kBatch][8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += f[i];
+    for (int b = 0; b < kBatch; ++b)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[b][i] = 0.0f;
+    for (int j = 0; j < slots; ++j) {
+      const uint16_t* src = g + row_dest[t * slots + j] * dim;
+      u32x4 v[kBatch];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b)
+        if (c0 + b * kWave < chunks) v[b] = ld16(src + (c0 + b * kWave) * 8);
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        if (c0 + b * kWave < chunks) {
+          float f[8];
+          unpack8(v[b], f);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[b][i] += f[i];
+        }
+      }
     }
-    store8_from_f32<kXF32>(gx, t * dim + c * 8, acc);
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b)
+      if (c0 + b * kWave < chunks) store8_from_f32<kXF32>(gx, t * dim + (c0 + b * kWave) * 8, acc[b]);
   }
 }
 
@@ -164,22 +212,38 @@ __global__ __launch_bounds__(kRowBlock) void combine_fwd_kernel(
   const int lane = threadIdx.x % kWave;
   const int chunks = static_cast<int>(dim / 8);
   const bool round = round_term != 0 && !kOutF32;  // rounding to fp32 is the identity
-  for (int c = lane; c < chunks; c += kWave) {
-    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    float acc[kBatch][8];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[b][i] = 0.0f;
     for (int e = 0; e < group; ++e) {
       const int64_t r = o * group + e;
-      const int64_t p = row_dest[r];
+      const uint16_t* src = y + row_dest[r] * dim;
       const float w = load_scalar(weights, r, w_dtype);
-      float f[8];
-      unpack8(ld16(y + p * dim + c * 8), f);
+      u32x4 v[kBatch];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        float term = f[i] * w;
-        if (round) term = round_bf16(term);
-        acc[i] += term;
+      for (int b = 0; b < kBatch; ++b)
+        if (c0 + b * kWave < chunks) v[b] = ld16(src + (c0 + b * kWave) * 8);
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        if (c0 + b * kWave < chunks) {
+          float f[8];
+          unpack8(v[b], f);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            float term = f[i] * w;
+            if (round) term = round_bf16(term);
+            acc[b][i] += term;
+          }
+        }
       }
     }
-    store8_from_f32<kOutF32>(out, o * dim + c * 8, acc);
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b)
+      if (c0 + b * kWave < chunks)
+        store8_from_f32<kOutF32>(out, o * dim + (c0 + b * kWave) * 8, acc[b]);
   }
 }
 
@@ -205,22 +269,92 @@ __global__ __launch_bounds__(kRowBlock) void combine_bwd_kernel(
   const float w = load_scalar(weights, src, w_dtype);
   const int64_t orow = src / group;
   float dot = 0.0f;
-  for (int c = lane; c < chunks; c += kWave) {
-    float go[8], o[8];
-    load8_as_f32<kGoF32>(gout, orow * dim + c * 8, go);
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    float go[kBatch][8];
+    u32x4 yv[kBatch];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = go[i] * w;
-    st16(dst + c * 8, pack8(o));
-    if (gw != nullptr) {
-      float f[8];
-      unpack8(ld16(y + p * dim + c * 8), f);
+    for (int b = 0; b < kBatch; ++b) {
+      const int c = c0 + b * kWave;
+      if (c < chunks) {
+        load8_as_f32<kGoF32>(gout, orow * dim + c * 8, go[b]);
+        if (gw != nullptr) yv[b] = ld16(y + p * dim + c * 8);
+      }
+    }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) dot += go[i] * f[i];
+    for (int b = 0; b < kBatch; ++b) {
+      const int c = c0 + b * kWave;
+      if (c < chunks) {
+        float o[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = go[b][i] * w;
+        st16(dst + c * 8, pack8(o));
+        if (gw != nullptr) {
+          float f[8];
+          unpack8(yv[b], f);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) dot += go[b][i] * f[i];
+        }
+      }
     }
   }
   if (gw != nullptr) {
     dot = wave_sum(dot);
     if (lane == 0) gw[src] = dot;
+  }
+}
+
+// Zero-fill of the padded rows that hold no assignment, for the source-major
+// kernels below: wavefront w looks at rows 64w .. 64w+63 (one per lane) and the
+// whole wavefront then clears each invalid one.
+__device__ __forceinline__ void zero_invalid_rows(const void* pad_valid, int valid_dtype,
+                                                  uint16_t* out, int64_t rows_pad, int64_t dim,
+                                                  int64_t w) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t p = w * kWave + lane;
+  const bool invalid = p < rows_pad && !load_valid(pad_valid, p, valid_dtype);
+  uint64_t todo = __ballot(invalid);
+  const int chunks = static_cast<int>(dim / 8);
+  const u32x4 zero = {0, 0, 0, 0};
+  while (todo != 0) {
+    const int l = __ffsll(static_cast<long long>(todo)) - 1;
+    todo &= todo - 1;
+    uint16_t* dst = out + (w * kWave + l) * dim;
+    for (int c = lane; c < chunks; c += kWave) st16(dst + c * 8, zero);
+  }
+}
+
+// Source-major dispatch: wavefront t reads token t once and writes it to the
+// padded rows of its `slots` assignments (row_dest), instead of every padded row
+// fetching its token: the activations cross HBM once, not once per slot.  An
+// assignment owns its destination only if the maps say so (a row dropped by a
+// capacity limit points at a slack row, which stays zero).  Wavefronts behind
+// the tokens clear the rows that hold no assignment.
+__global__ __launch_bounds__(kRowBlock) void dispatch_scatter_kernel(
+    const uint16_t* __restrict__ x, const int64_t* __restrict__ pad_token,
+    const void* __restrict__ pad_valid, int valid_dtype, const int64_t* __restrict__ row_dest,
+    uint16_t* __restrict__ out, int64_t rows_pad, int64_t num_tokens, int slots, int64_t dim) {
+  const int64_t t = wave_row();
+  if (t >= num_tokens) {
+    zero_invalid_rows(pad_valid, valid_dtype, out, rows_pad, dim, t - num_tokens);
+    return;
+  }
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const uint16_t* src = x + t * dim;
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    u32x4 v[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b)
+      if (c0 + b * kWave < chunks) v[b] = ld16(src + (c0 + b * kWave) * 8);
+    for (int j = 0; j < slots; ++j) {
+      const int64_t p = row_dest[t * slots + j];
+      if (p < 0 || p >= rows_pad || !load_valid(pad_valid, p, valid_dtype) || pad_token[p] != t)
+        continue;
+      uint16_t* dst = out + p * dim;
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b)
+        if (c0 + b * kWave < chunks) st16(dst + (c0 + b * kWave) * 8, v[b]);
+    }
   }
 }
 
@@ -238,20 +372,28 @@ extern "C" int nestor_hip_dispatch_rows_fwd(const void* x, int32_t x_dtype,
                                             const int64_t* pad_token,
                                             const void* pad_valid, int32_t valid_dtype,
                                             void* x_pad, int64_t rows_pad, int64_t dim,
-                                            void* stream) {
+                                            const int64_t* row_dest, int64_t num_tokens,
+                                            int32_t slots, void* stream) {
   if (!dtype_ok(x_dtype) || !dtype_ok(valid_dtype) || dim <= 0 || dim % 8 != 0 ||
-      rows_pad < 0)
+      rows_pad < 0 || (row_dest != nullptr && (num_tokens < 0 || slots <= 0)))
     return NESTOR_HIP_EINVAL;
   if (rows_pad == 0) return NESTOR_HIP_OK;
   if (!x || !pad_token || !pad_valid || !x_pad) return NESTOR_HIP_EINVAL;
   hipStream_t s = static_cast<hipStream_t>(stream);
   auto* out = static_cast<uint16_t*>(x_pad);
+  if (row_dest != nullptr && x_dtype == NESTOR_HIP_BF16) {
+    const int64_t waves = num_tokens + ceil_div(rows_pad, kWave);
+    hipLaunchKernelGGL(dispatch_scatter_kernel, dim3(row_blocks(waves)), dim3(kRowBlock), 0, s,
+                       static_cast<const uint16_t*>(x), pad_token, pad_valid, valid_dtype,
+                       row_dest, out, rows_pad, num_tokens, slots, dim);
+    return launch_status();
+  }
   if (x_dtype == NESTOR_HIP_F32)
-    hipLaunchKernelGGL(dispatch_fwd_kernel<true>, dim3(row_blocks(rows_pad)),
+    hipLaunchKernelGGL(dispatch_fwd_kernel<true>, dim3(row_blocks(ceil_div(rows_pad, kGatherRows))),
                        dim3(kRowBlock), 0, s, x, pad_token, pad_valid, valid_dtype, out,
                        rows_pad, dim);
   else
-    hipLaunchKernelGGL(dispatch_fwd_kernel<false>, dim3(row_blocks(rows_pad)),
+    hipLaunchKernelGGL(dispatch_fwd_kernel<false>, dim3(row_blocks(ceil_div(rows_pad, kGatherRows))),
                        dim3(kRowBlock), 0, s, x, pad_token, pad_valid, valid_dtype, out,
                        rows_pad, dim);
   return launch_status();

@@ -167,20 +167,27 @@ def _table_max_tiles(tile_table: Tensor) -> int:
 # Row moves
 # --------------------------------------------------------------------------
 @torch.library.custom_op(f"{_NS}::dispatch_rows_fwd", mutates_args=(), device_types="cuda")
-def dispatch_rows_fwd(x: Tensor, pad_token: Tensor, pad_valid: Tensor) -> Tensor:
+def dispatch_rows_fwd(
+    x: Tensor, pad_token: Tensor, pad_valid: Tensor, row_dest: Tensor | None = None,
+    slots: int = 0,
+) -> Tensor:
+    """``row_dest`` / ``slots`` (the inverse map) select the source-major kernel."""
+
     x = x.contiguous()
     rows_pad = pad_token.shape[0]
     out = torch.empty(rows_pad, x.shape[1], dtype=torch.bfloat16, device=x.device)
+    scatter = row_dest is not None and slots > 0
     _lib.call(
         "nestor_hip_dispatch_rows_fwd", _ptr(x), _code(x.dtype), _ptr(pad_token.contiguous()),
         _ptr(pad_valid.contiguous()), _code(pad_valid.dtype), _ptr(out), rows_pad,
-        x.shape[1], _stream(x),
+        x.shape[1], _ptr(row_dest.contiguous()) if scatter else None,
+        x.shape[0] if scatter else 0, slots if scatter else 0, _stream(x),
     )
     return out
 
 
 @dispatch_rows_fwd.register_fake
-def _(x, pad_token, pad_valid):
+def _(x, pad_token, pad_valid, row_dest=None, slots=0):
     return x.new_empty(pad_token.shape[0], x.shape[1], dtype=torch.bfloat16)
 
 
@@ -207,7 +214,7 @@ def _(grad_pad, row_dest, num_tokens, slots, x_dtype):
 def dispatch_rows_op(
     x: Tensor, pad_token: Tensor, pad_valid: Tensor, row_dest: Tensor, slots: int
 ) -> Tensor:
-    return dispatch_rows_fwd(x, pad_token, pad_valid)
+    return dispatch_rows_fwd(x, pad_token, pad_valid, row_dest, slots)
 
 
 @dispatch_rows_op.register_fake

@@ -133,6 +133,25 @@ def test_combine_rows_fwd_bwd(cuda, tokens, slots, group, banks, dim, out_dtype,
     torch.testing.assert_close(tw.grad.cpu().float(), gw_ref.to(w_dtype).float(), rtol=1e-2 if w_dtype == torch.bfloat16 else 1e-4, atol=1e-2 if w_dtype == torch.bfloat16 else 1e-3)
 
 
+@pytest.mark.parametrize("capacity", [0, 40])
+def test_source_major_and_row_major_kernels_agree(cuda, capacity):
+    """The two traversal orders of the dispatch gather write the same bits (with
+    and without rows dropped by a capacity limit)."""
+
+    from nestor_amd import ops
+    from nestor_amd.dispatch import dispatch_plan
+
+    tokens, slots, banks, dim = 700, 2, 9, 264
+    ids, _ = routing(11, tokens, slots, banks)
+    plan = dispatch_plan(ids.reshape(-1).to(cuda), banks, slots, torch.bfloat16, capacity)
+    x = torch.randn(tokens, dim, generator=gen(5)).to(torch.bfloat16).to(cuda)
+    a = ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid)
+    b = ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots)
+    assert torch.equal(a, b)
+    if capacity:
+        assert (plan.row_kept == 0).any()
+
+
 def test_identity_round_trip(cuda):
     """combine(dispatch(x)) with unit weights sums each token's ``slots`` copies."""
 

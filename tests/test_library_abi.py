@@ -40,7 +40,7 @@ def test_argument_checks_fail_before_any_launch():
 
     lib = _lib.load()
     null = ctypes.c_void_p(0)
-    assert lib.nestor_hip_dispatch_rows_fwd(null, 1, null, null, 1, null, 16, 12, null) == -22  # dim % 8
+    assert lib.nestor_hip_dispatch_rows_fwd(null, 1, null, null, 1, null, 16, 12, null, 0, 0, null) == -22  # dim % 8
     assert lib.nestor_hip_swiglu_fwd(null, null, null, 4, 20, 20, 20, null) == -22
     assert lib.nestor_hip_grouped_gemm_nn(null, null, null, 16, 12, 8, 1, null, 4, null) == -22
     assert lib.nestor_hip_router_topk(null, 1, null, 1, null, null, null, null, 4, 65, 1, 0, null) == -22
