@@ -577,10 +577,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
 // piece c ^ f(row); a contraction-major tile XORs the 32-byte column block with
 // the low bits of its row.  Fragment reads apply the same XOR.
 //
-// Requirements checked by the launcher: the contraction length is a multiple of
-// BK (row-tiled modes).  The weight gradient contracts over the rows of a
-// segment; rows behind the segment are redirected to the last padded row, which
-// is slack (all zero) in every padded tensor, so no step needs masking.
+// Requirement checked by the launcher: the contraction length is a multiple of
+// BK.  Row-tiled modes only; the weight gradient has its own kernel below.
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int STAGES_, int OCC_ = 1>
 struct DmaCfg {
   static constexpr int OCC = OCC_;  // workgroups resident per CU the register budget is sized for
@@ -663,11 +661,11 @@ __device__ __forceinline__ int nc_offset(int k, int n) {
 
 template <typename C, int kMode>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(GemmParams p) {
+  static_assert(kMode != kTN && kMode != kNNFp8W, "row-tiled bf16 modes");
   constexpr int kThreads = C::THREADS, kWaves = C::WAVES;
   extern __shared__ __align__(16) uint16_t lds[];
   constexpr int BM = C::BM, BN = C::BN, BK = C::BK;
   constexpr bool kUpGateFwd = kMode == kNNUpGate;
-  constexpr bool kAContig = kMode != kTN;
   constexpr bool kBContig = kMode == kNT || kMode == kNTUpGate;
   constexpr int kOutCols = kUpGateFwd ? BN / 2 : BN;
   // The forward up|gate tile is two contraction-major sub-tiles side by side
@@ -682,59 +680,37 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   const int wm = wave / C::WGN;
   const int wn = wave % C::WGN;
 
-  int bank, row0 = 0, nrows = BM;
-  int64_t n0, m0 = 0;
-  int64_t seg_begin = 0, seg_end = 0;
-  if constexpr (kMode == kTN) {
-    bank = blockIdx.z;
-    m0 = static_cast<int64_t>(blockIdx.y) * BM;
-    n0 = static_cast<int64_t>(blockIdx.x) * BN;
-    if (p.seg_start != nullptr) {
-      seg_begin = p.seg_start[bank];
-      seg_end = seg_begin + p.seg_count[bank];
-    } else {
-      seg_begin = bank == 0 ? 0 : p.offs[bank - 1];
-      seg_end = p.offs[bank];
-    }
-    if (seg_end > p.rows_pad) seg_end = p.rows_pad;
-  } else {
-    const int tile = blockIdx.x / p.n_tiles;
-    const int nt = blockIdx.x % p.n_tiles;
-    const int32_t* tt = p.tile_table;
-    if (tile >= tt[3 * p.max_tiles]) return;
-    bank = tt[tile];
-    row0 = tt[p.max_tiles + tile];
-    nrows = tt[2 * p.max_tiles + tile];
-    n0 = static_cast<int64_t>(nt) * kOutCols;
-    if (bank < 0) {
-      const u32x4 zero = {0, 0, 0, 0};
-      for (int c = tid; c < BM * (kOutCols / 8); c += kThreads) {
-        const int row = c / (kOutCols / 8);
-        const int64_t n = n0 + (c % (kOutCols / 8)) * 8;
-        if (row < nrows && n < p.N) {
-          const int64_t r = row0 + row;
-          if constexpr (kUpGateFwd) {
-            if (p.out != nullptr) {
-              st16(p.out + r * p.ldo + n, zero);
-              st16(p.out + r * p.ldo + p.N + n, zero);
-            }
-            st16(p.out2 + r * p.ldo2 + n, zero);
-          } else {
+  const int tile = blockIdx.x / p.n_tiles;
+  const int nt = blockIdx.x % p.n_tiles;
+  const int32_t* tt = p.tile_table;
+  if (tile >= tt[3 * p.max_tiles]) return;
+  const int bank = tt[tile];
+  const int row0 = tt[p.max_tiles + tile];
+  const int nrows = tt[2 * p.max_tiles + tile];
+  const int64_t n0 = static_cast<int64_t>(nt) * kOutCols;
+  if (bank < 0) {
+    const u32x4 zero = {0, 0, 0, 0};
+    for (int c = tid; c < BM * (kOutCols / 8); c += kThreads) {
+      const int row = c / (kOutCols / 8);
+      const int64_t n = n0 + (c % (kOutCols / 8)) * 8;
+      if (row < nrows && n < p.N) {
+        const int64_t r = row0 + row;
+        if constexpr (kUpGateFwd) {
+          if (p.out != nullptr) {
             st16(p.out + r * p.ldo + n, zero);
+            st16(p.out + r * p.ldo + p.N + n, zero);
           }
+          st16(p.out2 + r * p.ldo2 + n, zero);
+        } else {
+          st16(p.out + r * p.ldo + n, zero);
         }
       }
-      return;
     }
+    return;
   }
 
-  int num_kt, kt_per_phase = 1;
-  if constexpr (kMode == kTN) {
-    num_kt = seg_end > seg_begin ? static_cast<int>((seg_end - seg_begin + BK - 1) / BK) : 0;
-  } else {
-    kt_per_phase = static_cast<int>(p.K / BK);
-    num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
-  }
+  const int kt_per_phase = static_cast<int>(p.K / BK);
+  const int num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
 
   // Per-lane source offsets (elements) of every DMA instruction, relative to a
   // wavefront-uniform base that advances with the K step.
@@ -743,30 +719,17 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
 #pragma unroll
   for (int i = 0; i < C::A_CHUNKS; ++i) {
     const int ci = (wave + kWaves * i) * 64 + lane;  // 16-byte position in the tile
-    if constexpr (kAContig) {
-      constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
-      int row = ci / cpr;
-      const int c = (ci % cpr) ^ ((row / rp) % cpr);
-      row = row < last_row ? row : last_row;
-      offa[i] = static_cast<int64_t>(row0 + row) * p.lda + c * 8;
-    } else {
-      const int k = ci / (BM / 8);
-      const int c = (ci % (BM / 8)) ^ (4 * (k & 3));
-      int64_t m = m0 + c * 8;
-      m = m < p.M ? m : p.M - 8;
-      offa[i] = m;  // the row is added per step (it may be redirected)
-    }
+    constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
+    int row = ci / cpr;
+    const int c = (ci % cpr) ^ ((row / rp) % cpr);
+    row = row < last_row ? row : last_row;
+    offa[i] = static_cast<int64_t>(row0 + row) * p.lda + c * 8;
   }
 #pragma unroll
   for (int i = 0; i < C::B_CHUNKS; ++i) {
     const int blk = wave + kWaves * i;
     const int ci = blk * 64 + lane;
-    if constexpr (kMode == kTN) {
-      const int c = (ci % (BN / 8)) ^ (4 * ((ci / (BN / 8)) & 3));
-      int64_t n = n0 + c * 8;
-      n = n < p.N ? n : p.N - 8;
-      offb[i] = n;
-    } else if constexpr (kBContig) {
+    if constexpr (kBContig) {
       constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
       const int row = ci / cpr;
       const int c = (ci % cpr) ^ ((row / rp) % cpr);
@@ -784,7 +747,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       offb[i] = static_cast<int64_t>(k) * p.ldb + n;
     }
   }
-  const int64_t zero_row = p.rows_pad - 1;  // kTN: an all-zero row of every padded tensor
 
   // DMA instruction q (A pieces first, then B pieces) of K step kt into ring
   // stage `stage`.  Steps past the end re-fetch the last step: the extra tile
@@ -796,27 +758,14 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     uint16_t* sb = sa + C::A_ELEMS;
     if (q < C::A_CHUNKS) {
       const int i = q;
-      const uint16_t* src;
-      if constexpr (kAContig) {
-        src = p.a + offa[i] + static_cast<int64_t>(kt) * BK;
-      } else {
-        const int ci = (wave + kWaves * i) * 64 + lane;
-        int64_t r = seg_begin + static_cast<int64_t>(kt) * BK + ci / (BM / 8);
-        r = r < seg_end ? r : zero_row;
-        src = p.a + r * p.lda + offa[i];
-      }
+      const uint16_t* src = p.a + offa[i] + static_cast<int64_t>(kt) * BK;
       dma16(src, lds_byte_addr(sa + (wave + kWaves * i) * 512));
     } else {
       const int i = q - C::A_CHUNKS;
       const int blk = wave + kWaves * i;
       const uint16_t* src;
-      if constexpr (kMode == kTN) {
-        const int ci = blk * 64 + lane;
-        int64_t r = seg_begin + static_cast<int64_t>(kt) * BK + ci / (BN / 8);
-        r = r < seg_end ? r : zero_row;
-        src = reinterpret_cast<const uint16_t*>(p.b0) + r * p.ldb + offb[i];
-      } else if constexpr (kBContig) {
-        const int phase = kMode == kNTUpGate ? kt / kt_per_phase : 0;
+      if constexpr (kBContig) {
+        const int phase = (kMode == kNTUpGate && kt >= kt_per_phase) ? 1 : 0;
         const uint16_t* b = reinterpret_cast<const uint16_t*>(phase == 0 ? p.b0 : p.b1) +
                             bank * p.bank_stride;
         src = b + offb[i] + static_cast<int64_t>(kt - phase * kt_per_phase) * BK;
@@ -849,14 +798,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par, int mi_eff) __attribute__((always_inline)) {
     if (r >= 1 && r <= mi_eff) {
       const int i = r - 1;
-      if constexpr (kAContig) {
-        const int row = C::WTM * wm + 32 * i + kc_row;
-        fa[par][i] = *reinterpret_cast<const bf16x8*>(sa + kc_offset<BK>(row, 2 * kk + kc_piece));
-      } else {
-        const int k = 16 * kk + tr_krow;
-        const int n = C::WTM * wm + 32 * i + tr_col;
-        fa[par][i] = lds_read_tr_pair<BM>(sa + nc_offset<BM>(k, n));
-      }
+      const int row = C::WTM * wm + 32 * i + kc_row;
+      fa[par][i] = *reinterpret_cast<const bf16x8*>(sa + kc_offset<BK>(row, 2 * kk + kc_piece));
     } else {
       const int j = r == 0 ? 0 : r - mi_eff;
       if constexpr (kBContig) {
@@ -960,11 +903,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     __builtin_amdgcn_sched_barrier(0);
     // Row blocks in use: only tiles with a single row of wavefronts can skip.
     int mi_eff = C::MI;
-    if constexpr (C::WGM == 1 && kMode != kTN && C::MI == 4) {
+    if constexpr (C::WGM == 1 && C::MI == 4) {
       mi_eff = (nrows + 31) >> 5;
       mi_eff = mi_eff < 1 ? 1 : (mi_eff > 4 ? 4 : mi_eff);
     }
-    if constexpr (C::WGM == 1 && kMode != kTN && C::MI == 4) {
+    if constexpr (C::WGM == 1 && C::MI == 4) {
       switch (mi_eff) {
         case 1: k_loop(std::integral_constant<int, 1>{}); break;
         case 2: k_loop(std::integral_constant<int, 2>{}); break;
@@ -1027,16 +970,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
         st16(p.out2 + r * p.ldo2 + n, pack8(h));
       }
     }
-  } else if constexpr (kMode == kTN) {
-    uint16_t* out = p.out + bank * p.bank_stride;
-    for (int c = tid; c < BM * (BN / 8); c += kThreads) {
-      const int64_t m = m0 + c / (BN / 8);
-      const int64_t n = n0 + (c % (BN / 8)) * 8;
-      if (m < p.M && n < p.N)
-        st16(out + m * p.ldo + n,
-             *reinterpret_cast<const u32x4*>(stage + (c / (BN / 8)) * C::STAGE_LD +
-                                             (c % (BN / 8)) * 8));
-    }
   } else {
     for (int c = tid; c < BM * (BN / 8); c += kThreads) {
       const int row = c / (BN / 8);
@@ -1046,324 +979,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
              *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + (c % (BN / 8)) * 8));
     }
   }
-}
-
-// ---------------------------------------------------------------------------
-// Persistent variant of the direct-to-LDS kernel for the row-tiled modes.  One
-// workgroup per CU walks a list of output tiles; the LDS ring never drains
-// between tiles, so the fetch of the next tile's first K steps overlaps the
-// last K steps and the epilogue of the current one, and the accumulators leave
-// through a per-wavefront staging area that needs no workgroup barrier.
-//
-// Work order: output tiles are numbered so that 32 consecutive numbers form a
-// 4 (row tiles) x 8 (column tiles) rectangle, and consecutive groups of 32 go
-// to consecutive XCDs (workgroup b runs on XCD b % 8): the 32 CUs of one XCD
-// work on one rectangle at a time and share its 4 activation and 8 weight
-// panels through that XCD's L2.
-template <typename C>
-struct PersLayout {
-  static constexpr int kRingElems = C::kStages * (C::A_ELEMS + C::B_ELEMS);
-  static constexpr int kEpiLd = C::WTN + 8;
-  static constexpr int kEpiElems = 32 * kEpiLd;  // one 32-row slab per wavefront
-  static constexpr size_t LDS_BYTES = sizeof(uint16_t) * (kRingElems + C::WAVES * kEpiElems);
-};
-
-template <typename C, int kMode>
-__global__ __launch_bounds__(C::THREADS, 1) void grouped_gemm_persistent_kernel(GemmParams p) {
-  static_assert(kMode == kNN || kMode == kNT || kMode == kNNUpGate || kMode == kNTUpGate, "row-tiled");
-  constexpr int kWaves = C::WAVES;
-  extern __shared__ __align__(16) uint16_t lds[];
-  constexpr int BM = C::BM, BN = C::BN, BK = C::BK, S = C::kStages;
-  constexpr bool kUpGateFwd = kMode == kNNUpGate;
-  constexpr bool kBContig = kMode == kNT || kMode == kNTUpGate;
-  constexpr int kOutCols = kUpGateFwd ? BN / 2 : BN;
-  constexpr int kSub = kUpGateFwd ? 2 : 1;
-  constexpr int BW = BN / kSub;
-  constexpr int kStageElems = C::A_ELEMS + C::B_ELEMS;
-  constexpr int kLoads = C::A_CHUNKS + C::B_CHUNKS;
-  constexpr int kLoadsPerBlock = kLoads / C::KK;
-  constexpr int kReads = C::MI + C::NJ;
-  constexpr int kMfma = C::MI * C::NJ;
-  using L = PersLayout<C>;
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / C::WGN;
-  const int wn = wave % C::WGN;
-
-  // ---- work list -----------------------------------------------------------
-  const int32_t* tt = p.tile_table;
-  const int num_rt = tt[3 * p.max_tiles + 1];  // row tiles of BM rows
-  const int n_tiles = p.n_tiles;
-  const int per_xcd = gridDim.x >> 3;
-  const int xcd = blockIdx.x & 7;
-  const int slot = blockIdx.x >> 3;
-  const bool rect = per_xcd == 32 && (n_tiles & 7) == 0;
-  const int band_items = 4 * n_tiles;
-  const int w_end = rect ? ((num_rt + 3) >> 2) * band_items : num_rt * n_tiles;
-  // i-th item of this workgroup -> (row tile, column tile); false past the end.
-  auto decode = [&](int i, int& mt, int& nt) __attribute__((always_inline)) -> bool {
-    const int w = (i * 8 + xcd) * per_xcd + slot;
-    if (w >= w_end) return false;
-    if (rect) {
-      const int band = w / band_items;
-      const int r = w - band * band_items;
-      mt = band * 4 + ((r & 31) >> 3);
-      nt = (r >> 5) * 8 + (r & 7);
-    } else {
-      mt = w / n_tiles;
-      nt = w - mt * n_tiles;
-    }
-    return mt < num_rt;
-  };
-  int count = 0;
-  {
-    int mt, nt;
-    while (decode(count, mt, nt)) ++count;
-  }
-  if (count == 0) return;
-  const int kt_per_phase = static_cast<int>(p.K / BK);
-  const int num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
-
-  // ---- load cursor -----------------------------------------------------------
-  int64_t offa[C::A_CHUNKS], offb[C::B_CHUNKS];
-  int l_item = 0, l_kt = 0, l_stage = 0;
-  auto set_load_item = [&](int i) __attribute__((always_inline)) {
-    int mt, nt;
-    decode(i, mt, nt);
-    const int bank = tt[mt];
-    const int row0 = tt[p.max_tiles + mt];
-    const int nrows = tt[2 * p.max_tiles + mt];
-    const int64_t n0 = static_cast<int64_t>(nt) * kOutCols;
-    const int last_row = nrows - 1;
-#pragma unroll
-    for (int c = 0; c < C::A_CHUNKS; ++c) {
-      const int ci = (wave + kWaves * c) * 64 + lane;
-      constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
-      int row = ci / cpr;
-      const int pc = (ci % cpr) ^ ((row / rp) % cpr);
-      row = row < last_row ? row : last_row;
-      offa[c] = static_cast<int64_t>(row0 + row) * p.lda + pc * 8;
-    }
-#pragma unroll
-    for (int c = 0; c < C::B_CHUNKS; ++c) {
-      const int ci = (wave + kWaves * c) * 64 + lane;
-      if constexpr (kBContig) {
-        constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
-        const int row = ci / cpr;
-        const int pc = (ci % cpr) ^ ((row / rp) % cpr);
-        int64_t n = n0 + row;
-        n = n < p.N ? n : p.N - 1;
-        offb[c] = bank * p.bank_stride + n * p.ldb + pc * 8;
-      } else {
-        constexpr int kPerSub = BK * BW / 8;
-        const int cs = ci % kPerSub;
-        const int k = cs / (BW / 8);
-        const int pc = (cs % (BW / 8)) ^ (4 * (k & 3));
-        int64_t n = n0 + pc * 8;
-        n = n < p.N ? n : p.N - 8;
-        offb[c] = bank * p.bank_stride + static_cast<int64_t>(k) * p.ldb + n;
-      }
-    }
-  };
-  // DMA instruction q of the cursor's K step into the cursor's ring stage.
-  auto issue_one = [&](int q) __attribute__((always_inline)) {
-    uint16_t* sa = lds + l_stage * kStageElems;
-    uint16_t* sb = sa + C::A_ELEMS;
-    if (q < C::A_CHUNKS) {
-      const uint16_t* src = p.a + offa[q] + static_cast<int64_t>(l_kt) * BK;
-      dma16(src, lds_byte_addr(sa + (wave + kWaves * q) * 512));
-    } else {
-      const int c = q - C::A_CHUNKS;
-      const int blk = wave + kWaves * c;
-      const uint16_t* src;
-      if constexpr (kBContig) {
-        const int phase = (kMode == kNTUpGate && l_kt >= kt_per_phase) ? 1 : 0;
-        src = reinterpret_cast<const uint16_t*>(phase == 0 ? p.b0 : p.b1) + offb[c] +
-              static_cast<int64_t>(l_kt - phase * kt_per_phase) * BK;
-      } else {
-        constexpr int kBlkPerSub = BK * BW / 8 / 64;
-        src = reinterpret_cast<const uint16_t*>((kSub == 2 && blk >= kBlkPerSub) ? p.b1 : p.b0) +
-              offb[c] + static_cast<int64_t>(l_kt) * BK * p.ldb;
-      }
-      dma16(src, lds_byte_addr(sb + blk * 512));
-    }
-  };
-  // Next K step of the work list; past the end the last step is fetched again
-  // (into a stage nobody reads), which keeps the vmcnt bookkeeping uniform.
-  auto advance = [&]() __attribute__((always_inline)) {
-    l_stage = l_stage == S - 1 ? 0 : l_stage + 1;
-    if (l_kt + 1 < num_kt) {
-      ++l_kt;
-    } else if (l_item + 1 < count) {
-      ++l_item;
-      l_kt = 0;
-      set_load_item(l_item);
-    }
-  };
-
-  // ---- fragments -------------------------------------------------------------
-  f32x16 acc[C::MI][C::NJ];
-  const int kc_row = lane & 31, kc_piece = lane >> 5;
-  const int tr_krow = 8 * (lane >> 5) + ((lane & 15) >> 2);
-  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-  // Column of B fragment j inside the B tile.  Forward up|gate: each wavefront
-  // owns the same WTN/2 output columns of the up and of the gate sub-tile, so
-  // its epilogue finds both factors of a hidden element in its own registers.
-  auto b_col = [&](int j, int& sub) __attribute__((always_inline)) -> int {
-    if constexpr (kUpGateFwd) {
-      sub = j / (C::NJ / 2);
-      return (C::WTN / 2) * wn + 32 * (j % (C::NJ / 2));
-    } else {
-      sub = 0;
-      return C::WTN * wn + 32 * j;
-    }
-  };
-  bf16x8 fa[2][C::MI], fb[2][C::NJ];
-  auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par) __attribute__((always_inline)) {
-    if (r >= 1 && r <= C::MI) {
-      const int i = r - 1;
-      const int row = C::WTM * wm + 32 * i + kc_row;
-      fa[par][i] = *reinterpret_cast<const bf16x8*>(sa + kc_offset<BK>(row, 2 * kk + kc_piece));
-    } else {
-      const int j = r == 0 ? 0 : r - C::MI;
-      int sub;
-      const int col = b_col(j, sub);
-      if constexpr (kBContig) {
-        const int row = col + kc_row;
-        fb[par][j] = *reinterpret_cast<const bf16x8*>(sb + kc_offset<BK>(row, 2 * kk + kc_piece));
-      } else {
-        const uint16_t* base = sb + sub * (BK * BW);
-        const int k = 16 * kk + tr_krow;
-        fb[par][j] = lds_read_tr_pair<BW>(base + nc_offset<BW>(k, col + tr_col));
-      }
-    }
-  };
-  auto mfma_block = [&](int par, const uint16_t* ra, const uint16_t* rb, int rkk, int l0) __attribute__((always_inline)) {
-    static_for<kMfma>([&](auto mc) __attribute__((always_inline)) {
-      constexpr int m = decltype(mc)::value;
-#pragma unroll
-      for (int r = m * kReads / kMfma; r < (m + 1) * kReads / kMfma; ++r)
-        read_one(ra, rb, rkk, r, par ^ 1);
-#pragma unroll
-      for (int q = m * kLoadsPerBlock / kMfma; q < (m + 1) * kLoadsPerBlock / kMfma; ++q)
-        issue_one(l0 + q);
-      constexpr int j = m / C::MI, i = m % C::MI;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[par][j], fa[par][i], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    });
-  };
-
-  // ---- epilogue of one output tile, per wavefront -----------------------------
-  uint16_t* epi = lds + L::kRingElems + wave * L::kEpiElems;
-  auto epilogue = [&](int item) __attribute__((always_inline)) {
-    int mt, nt;
-    decode(item, mt, nt);
-    const int row0 = tt[p.max_tiles + mt];
-    const int nrows = tt[2 * p.max_tiles + mt];
-    const int64_t n0 = static_cast<int64_t>(nt) * kOutCols;
-#pragma unroll
-    for (int i = 0; i < C::MI; ++i) {
-      __builtin_amdgcn_sched_barrier(0);  // one slab's worth of registers at a time
-#pragma unroll
-      for (int j = 0; j < C::NJ; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = 32 * j + 8 * q + 4 * (lane >> 5);
-          // Read the accumulators where they are used: left to the compiler, all
-          // 256 reads move to the top of the epilogue and spill.
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][4 * q + e]));
-          u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-          *reinterpret_cast<u32x2*>(epi + (lane & 31) * L::kEpiLd + n) = packed;
-        }
-      // same wavefront wrote and reads: program order is enough
-      if constexpr (kUpGateFwd) {
-        constexpr int kHalf = C::WTN / 2;          // output columns of this wavefront
-        constexpr int kCpr = kHalf / 8;            // 16-byte pieces per row
-#pragma unroll
-        for (int c = lane; c < 32 * kCpr; c += 64) {
-          const int r = c / kCpr, pc = c % kCpr;
-          const int row = C::WTM * wm + 32 * i + r;
-          const int64_t n = n0 + kHalf * wn + pc * 8;
-          const u32x4 up = *reinterpret_cast<const u32x4*>(epi + r * L::kEpiLd + pc * 8);
-          const u32x4 gate = *reinterpret_cast<const u32x4*>(epi + r * L::kEpiLd + kHalf + pc * 8);
-          if (row < nrows && n < p.N) {
-            const int64_t gr = row0 + row;
-            if (p.out != nullptr) {
-              st16(p.out + gr * p.ldo + n, up);
-              st16(p.out + gr * p.ldo + p.N + n, gate);
-            }
-            float u[8], g[8], h[8];
-            unpack8(up, u);
-            unpack8(gate, g);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) h[e] = round_bf16(g[e] / (1.0f + __expf(-g[e]))) * u[e];
-            st16(p.out2 + gr * p.ldo2 + n, pack8(h));
-          }
-        }
-      } else {
-        constexpr int kCpr = C::WTN / 8;
-#pragma unroll
-        for (int c = lane; c < 32 * kCpr; c += 64) {
-          const int r = c / kCpr, pc = c % kCpr;
-          const int row = C::WTM * wm + 32 * i + r;
-          const int64_t n = n0 + C::WTN * wn + pc * 8;
-          const u32x4 v = *reinterpret_cast<const u32x4*>(epi + r * L::kEpiLd + pc * 8);
-          if (row < nrows && n < p.N) st16(p.out + (row0 + row) * p.ldo + n, v);
-        }
-      }
-    }
-  };
-
-  // ---- pipeline ----------------------------------------------------------------
-  set_load_item(0);
-#pragma unroll
-  for (int t = 0; t + 1 < S; ++t) {
-#pragma unroll
-    for (int q = 0; q < kLoads; ++q) issue_one(q);
-    advance();
-  }
-#pragma unroll
-  for (int q = 0; q < kLoadsPerBlock; ++q) issue_one(q);
-  wait_vmcnt<(S - 2) * kLoads + kLoadsPerBlock>();
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int r = 0; r < kReads; ++r) read_one(lds, lds + C::A_ELEMS, 0, r, 0);
-
-  int cur = 0;
-  for (int item = 0; item < count; ++item) {
-#pragma unroll
-    for (int i = 0; i < C::MI; ++i)
-#pragma unroll
-      for (int j = 0; j < C::NJ; ++j)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-    for (int kt = 0; kt < num_kt; ++kt) {
-      const int nxt = cur == S - 1 ? 0 : cur + 1;
-      const uint16_t* sa = lds + cur * kStageElems;
-      const uint16_t* sb = sa + C::A_ELEMS;
-      const uint16_t* na = lds + nxt * kStageElems;
-      const uint16_t* nb = na + C::A_ELEMS;
-#pragma unroll
-      for (int kk = 0; kk + 1 < C::KK; ++kk)
-        mfma_block(kk & 1, sa, sb, kk + 1, (kk + 1) * kLoadsPerBlock);
-      advance();
-      // The next K step has landed once only the later steps' transfers are
-      // outstanding.
-      wait_vmcnt<(S - 2) * kLoads>();
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_block((C::KK - 1) & 1, na, nb, 0, 0);
-      cur = nxt;
-    }
-    epilogue(item);
-  }
-  wait_vmcnt<0>();
 }
 
 // ---------------------------------------------------------------------------
@@ -1727,10 +1342,7 @@ int launch_rows(GemmParams p, void* stream) {
 
 using DmaXWide = DmaCfg<128, 512, 32, 1, 4, 3>;   // wavefront tile 128 x 128, 3-stage DMA ring
 using DmaWide = DmaCfg<128, 256, 64, 2, 2, 3>;    // wavefront tile 64 x 128
-using DmaSquare = DmaCfg<256, 256, 32, 2, 2, 3>;  // weight gradient
-using DmaWide2 = DmaCfg<128, 256, 32, 2, 2, 3, 2>;  // two workgroups per CU
 using WgradPers = DmaCfg<256, 256, 32, 2, 2, 3>;  // persistent weight gradient
-using DmaSquare8 = DmaCfg<256, 256, 32, 2, 4, 4>;  // 8 wavefronts, tile 128 x 64 each
 
 template <typename C, int kMode>
 int launch_rows_dma(GemmParams p, void* stream) {
@@ -1747,28 +1359,6 @@ int launch_rows_dma(GemmParams p, void* stream) {
   }
   hipLaunchKernelGGL((grouped_gemm_dma_kernel<C, kMode>), dim3(static_cast<unsigned>(blocks)),
                      dim3(C::THREADS), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
-  return launch_status();
-}
-
-using PersSquare = DmaCfg<256, 256, 32, 2, 2, 3>;
-
-template <typename C, int kMode>
-int launch_rows_persistent(GemmParams p, void* stream) {
-  constexpr int out_cols = kMode == kNNUpGate ? C::BN / 2 : C::BN;
-  p.n_tiles = static_cast<int>(ceil_div(p.N, out_cols));
-  static int num_cus = 0;
-  if (num_cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-      return NESTOR_HIP_ELAUNCH;
-    num_cus = prop.multiProcessorCount / 8 * 8;
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_persistent_kernel<C, kMode>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(PersLayout<C>::LDS_BYTES));
-  }
-  hipLaunchKernelGGL((grouped_gemm_persistent_kernel<C, kMode>), dim3(static_cast<unsigned>(num_cus)),
-                     dim3(C::THREADS), PersLayout<C>::LDS_BYTES, static_cast<hipStream_t>(stream), p);
   return launch_status();
 }
 
@@ -1791,9 +1381,6 @@ int dispatch_rows_gemm(const GemmParams& p, void* stream) {
     // Direct-to-LDS variants: whole K steps only.
     if (cfg == 3 && width >= 512 && p.K % 32 == 0) return launch_rows_dma<DmaXWide, kMode>(p, stream);
     if (cfg == 4 && width >= 256 && p.K % 64 == 0) return launch_rows_dma<DmaWide, kMode>(p, stream);
-    if (cfg == 5 && width >= 256 && p.K % 32 == 0) return launch_rows_dma<DmaSquare, kMode>(p, stream);
-    if (cfg == 6 && width >= 256 && p.K % 32 == 0) return launch_rows_dma<DmaSquare8, kMode>(p, stream);
-    if (cfg == 7 && width >= 256 && p.K % 32 == 0) return launch_rows_dma<DmaWide2, kMode>(p, stream);
   }
   if (cfg >= 3) cfg = 2;
   if (cfg == 2 && width < 512) cfg = 1;
@@ -1996,23 +1583,6 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
     }
   }
   if (cfg == 5) cfg = 3;
-  if (cfg == 4 && M >= 256 && N >= 256) {
-    static bool configured = false;
-    if (!configured) {
-      (void)hipFuncSetAttribute(
-          reinterpret_cast<const void*>(grouped_gemm_dma_kernel<DmaSquare, kTN>),
-          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(DmaSquare::LDS_BYTES));
-      configured = true;
-    }
-    const int64_t my = ceil_div(M, DmaSquare::BM);
-    if (my > 65535) return NESTOR_HIP_ERANGE;
-    hipLaunchKernelGGL((grouped_gemm_dma_kernel<DmaSquare, kTN>),
-                       dim3(static_cast<unsigned>(ceil_div(N, DmaSquare::BN)),
-                            static_cast<unsigned>(my), static_cast<unsigned>(num_banks)),
-                       dim3(DmaSquare::THREADS), DmaSquare::LDS_BYTES, static_cast<hipStream_t>(stream), p);
-    return launch_status();
-  }
-  if (cfg == 4) cfg = 3;
   switch (cfg) {
     case 3: return launch_wgrad<CfgSquare>(p, num_banks, stream);
     case 1: return launch_wgrad<CfgWide>(p, num_banks, stream);
