@@ -92,6 +92,7 @@ struct GemmParams {
   const int32_t* tile_table;
   int64_t max_tiles;
   int n_tiles;
+  int tile_group;       // row tiles per XCD group in the grouped tile order (0: plain order)
   // kTN segment description
   int64_t rows_pad;
   const int32_t* offs;
@@ -688,15 +689,14 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   // +3..5 %).  The GEMMs that stream wide weight panels once do better when all
   // XCDs walk the same expert at the same time, each on its own column tiles
   // (plain order, column tile fastest).
-  constexpr bool kGroupTiles = kMode == kNN || kMode == kNTUpGate;
   int tile, nt;
-  if constexpr (kGroupTiles) {
+  if (p.tile_group > 0) {
     const int xcd = blockIdx.x & 7;
     const int local = blockIdx.x >> 3;
-    const int per_group = 4 * p.n_tiles;
+    const int per_group = p.tile_group * p.n_tiles;
     const int group = local / per_group;
     const int within = local - group * per_group;
-    tile = (group * 8 + xcd) * 4 + within / p.n_tiles;
+    tile = (group * 8 + xcd) * p.tile_group + within / p.n_tiles;
     nt = within % p.n_tiles;
   } else {
     tile = blockIdx.x / p.n_tiles;
@@ -1368,8 +1368,11 @@ template <typename C, int kMode>
 int launch_rows_dma(GemmParams p, void* stream) {
   constexpr int out_cols = kMode == kNNUpGate ? C::BN / 2 : C::BN;
   p.n_tiles = static_cast<int>(ceil_div(p.N, out_cols));
-  // whole groups of 4 row tiles per XCD (see the kernel's tile mapping)
-  const int64_t blocks = ceil_div(p.max_tiles, 32) * 32 * p.n_tiles;
+  static const int forced_group = config_choice("NESTOR_HIP_TILE_GROUP", -1);
+  p.tile_group = forced_group >= 0 ? forced_group : ((kMode == kNN || kMode == kNTUpGate) ? 4 : 0);
+  // whole groups of row tiles per XCD (see the kernel's tile mapping)
+  const int64_t gran = p.tile_group > 0 ? 8 * p.tile_group : 1;
+  const int64_t blocks = ceil_div(p.max_tiles, gran) * gran * p.n_tiles;
   if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
   static bool configured = false;
   if (!configured) {
