@@ -210,7 +210,43 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
         return ids.reshape(num_tokens, k_a * k_q), weights.reshape(num_tokens, k_a * k_q), selected
 
     # -- routing -------------------------------------------------------------
+    def _fused_head_scores(self, x: Tensor):
+        """Scores of the public router, the ``G`` private routers and the path gate
+        from ONE GEMM over ``x`` when all of them are single linear maps: they read
+        the same rows, and at production widths each separate skinny GEMM costs a
+        full pass over the activations (forward) and one more for its input
+        gradient (backward).  ``None`` when the heads cannot be fused."""
+
+        if not (self.batched_routers and self.public_router is not None):
+            return None
+        heads = [self.public_router.score_mlp, *[r.score_mlp for r in self.private_routers]]
+        if any(len(h.layers) != 1 for h in heads):
+            return None
+        layers = [h.layers[0] for h in heads] + [self.path_gate]
+        weight = torch.cat([l.weight for l in layers])
+        bias = None
+        if any(l.bias is not None for l in layers):
+            bias = torch.cat([
+                l.bias if l.bias is not None else l.weight.new_zeros(l.weight.shape[0])
+                for l in layers
+            ])
+        out = F.linear(x.reshape(-1, self.dim), weight, bias)
+        n_pub = layers[0].weight.shape[0]
+        n_priv = sum(l.weight.shape[0] for l in layers[1:-1])
+        return (out[:, :n_pub].reshape(*x.shape[:-1], n_pub), out[:, n_pub:n_pub + n_priv],
+                out[:, n_pub + n_priv:].reshape(*x.shape[:-1], -1))
+
     def _route(self, x: Tensor, valid: Tensor, group_active: Tensor):
+        fused = self._fused_head_scores(x)
+        self._path_logits = None
+        if fused is not None:
+            pub_scores, priv_scores, self._path_logits = fused
+            public_output = self.public_router(x, valid, scores=pub_scores)
+            outs, gates, choices = route_private_batched(
+                list(self.private_routers), x, valid, group_active, training=self.training,
+                scores=priv_scores,
+            )
+            return public_output, outs, (gates, choices)
         public_output = self.public_router(x, valid) if self.public_router is not None else None
         if self.batched_routers:
             outs, gates, choices = route_private_batched(
@@ -239,7 +275,11 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
                           self.private_top_k)
 
     def _path_weights(self, x: Tensor) -> Tensor:
-        return F.softmax(self.path_gate(x).float(), dim=-1).to(x.dtype)
+        logits = getattr(self, "_path_logits", None)
+        self._path_logits = None
+        if logits is None:
+            logits = self.path_gate(x)
+        return F.softmax(logits.float(), dim=-1).to(x.dtype)
 
     def _prologue(self, x: Tensor, valid: Tensor, group_gates: Tensor, group_active: Tensor):
         flat_x = x.reshape(-1, self.dim)

@@ -122,8 +122,13 @@ class Router(nn.Module):
         self.noise_mlp = None
         self.register_buffer("choice_bias", torch.zeros(num_choices))
 
-    def forward(self, x: Tensor, valid_token_mask: Tensor, noise: Tensor | None = None) -> RouterOutput:
-        scores = self.score_mlp(x)
+    def forward(self, x: Tensor, valid_token_mask: Tensor, noise: Tensor | None = None,
+                scores: Tensor | None = None) -> RouterOutput:
+        """``scores``: the score head's output when the caller already computed it
+        (one GEMM for several heads that read the same rows)."""
+
+        if scores is None:
+            scores = self.score_mlp(x)
         probs, topk, gates = route_scores(
             scores, self.choice_bias, self.num_choices_per_token, self.gate_mode, valid_token_mask
         )
@@ -168,18 +173,19 @@ def batched_mlp(x: Tensor, mlps: list[ScoreMLP]) -> Tensor:
 
 def route_private_batched(
     routers: list[Router], x: Tensor, valid_token_mask: Tensor, group_active_mask: Tensor,
-    training: bool, noise: Tensor | None = None,
+    training: bool, noise: Tensor | None = None, scores: Tensor | None = None,
 ) -> tuple[list[RouterOutput], Tensor, Tensor]:
     """All ``G`` private routers of a layer in one pass: per-group outputs (views
     of the stacked tensors, masked to ``valid & member``), stacked gates
-    ``[B, S, G, Q]`` and stacked choices ``[B, S, G, k]``."""
+    ``[B, S, G, Q]`` and stacked choices ``[B, S, G, k]``.  ``scores``
+    (``[B*S, G*Q]``, head-major) skips the score GEMM when the caller has it."""
 
     first = routers[0]
     groups = len(routers)
     batch, seq, dim = x.shape
-    scores = batched_mlp(x.reshape(batch * seq, dim), [r.score_mlp for r in routers]).view(
-        batch, seq, groups, first.num_choices
-    )
+    if scores is None:
+        scores = batched_mlp(x.reshape(batch * seq, dim), [r.score_mlp for r in routers])
+    scores = scores.reshape(batch, seq, groups, first.num_choices)
     bias = torch.stack([r.choice_bias for r in routers])
     member = valid_token_mask.unsqueeze(-1) & group_active_mask
     probs, topk, gates = route_scores(
