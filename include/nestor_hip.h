@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 2
+#define NESTOR_HIP_ABI_VERSION 3
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -259,6 +259,25 @@ int nestor_hip_router_topk(
     float* softmax_probs, int64_t* topk_indices, void* gates,
     int64_t n, int32_t num_choices, int32_t top_k, int32_t gate_mode,
     void* stream);
+
+/* ------------------------------------------------------------------------
+ * Path mix of the pool's summed layout: update = alpha_public * public_update +
+ * alpha_private * private_update with alpha = softmax of the 2-logit path gate
+ * (nestor/backbones/expert_pools.py:1103-1114).  All tensors share `dtype`
+ * (bf16 or fp32, the pool input's); each product and the sum are rounded to it,
+ * as the eager expression rounds them.  alpha is [num_tokens, 2].
+ * ---------------------------------------------------------------------- */
+int nestor_hip_path_mix_fwd(
+    const void* public_update, const void* private_update, const void* alpha,
+    void* out, int32_t dtype, int64_t num_tokens, int64_t dim, void* stream);
+/* grad_public = g*alpha[:,0], grad_private = g*alpha[:,1],
+ * grad_alpha[t,0] = sum_d g*public, grad_alpha[t,1] = sum_d g*private (terms
+ * rounded to `dtype`, fp32 sum, one final rounding): what autograd derives from
+ * the expression above. */
+int nestor_hip_path_mix_bwd(
+    const void* grad_out, const void* public_update, const void* private_update,
+    const void* alpha, void* grad_public, void* grad_private, void* grad_alpha,
+    int32_t dtype, int64_t num_tokens, int64_t dim, void* stream);
 
 #ifdef __cplusplus
 }

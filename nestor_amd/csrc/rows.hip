@@ -303,6 +303,108 @@ __global__ __launch_bounds__(kRowBlock) void combine_bwd_kernel(
   }
 }
 
+// Rounding of one eager op's result: bf16 results are rounded from the fp32
+// value, fp32 results are the fp32 value.
+template <bool kF32>
+__device__ __forceinline__ float round_to(float v) {
+  if constexpr (kF32) return v;
+  return round_bf16(v);
+}
+
+// update[t,:] = alpha[t,0]*pub[t,:] + alpha[t,1]*priv[t,:] with the roundings of
+// the eager expression: each product, then the sum.
+template <bool kF32>
+__global__ __launch_bounds__(kRowBlock) void path_mix_fwd_kernel(
+    const void* __restrict__ pub, const void* __restrict__ priv,
+    const void* __restrict__ alpha, void* __restrict__ out, int64_t num_tokens, int64_t dim) {
+#pragma clang fp contract(off)  // a fused multiply-add would skip the product's rounding
+  const int64_t t = wave_row();
+  if (t >= num_tokens) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const int dt = kF32 ? NESTOR_HIP_F32 : NESTOR_HIP_BF16;
+  const float a0 = load_scalar(alpha, 2 * t, dt);
+  const float a1 = load_scalar(alpha, 2 * t + 1, dt);
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    float u[kBatch][8], v[kBatch][8];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int c = c0 + b * kWave;
+      if (c < chunks) {
+        load8_as_f32<kF32>(pub, t * dim + c * 8, u[b]);
+        load8_as_f32<kF32>(priv, t * dim + c * 8, v[b]);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int c = c0 + b * kWave;
+      if (c < chunks) {
+        float o[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          o[i] = round_to<kF32>(a0 * u[b][i]) + round_to<kF32>(a1 * v[b][i]);
+        store8_from_f32<kF32>(out, t * dim + c * 8, o);
+      }
+    }
+  }
+}
+
+// g_pub = g*alpha0, g_priv = g*alpha1 (rounded), g_alpha[t,0] = sum_d round(g*pub),
+// g_alpha[t,1] = sum_d round(g*priv): fp32 sums in a fixed order, rounded once.
+template <bool kF32>
+__global__ __launch_bounds__(kRowBlock) void path_mix_bwd_kernel(
+    const void* __restrict__ g, const void* __restrict__ pub, const void* __restrict__ priv,
+    const void* __restrict__ alpha, void* __restrict__ g_pub, void* __restrict__ g_priv,
+    void* __restrict__ g_alpha, int64_t num_tokens, int64_t dim) {
+#pragma clang fp contract(off)  // a fused multiply-add would skip the product's rounding
+  const int64_t t = wave_row();
+  if (t >= num_tokens) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const int dt = kF32 ? NESTOR_HIP_F32 : NESTOR_HIP_BF16;
+  const float a0 = load_scalar(alpha, 2 * t, dt);
+  const float a1 = load_scalar(alpha, 2 * t + 1, dt);
+  float dot0 = 0.0f, dot1 = 0.0f;
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    float go[kBatch][8], u[kBatch][8], v[kBatch][8];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int c = c0 + b * kWave;
+      if (c < chunks) {
+        load8_as_f32<kF32>(g, t * dim + c * 8, go[b]);
+        load8_as_f32<kF32>(pub, t * dim + c * 8, u[b]);
+        load8_as_f32<kF32>(priv, t * dim + c * 8, v[b]);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int c = c0 + b * kWave;
+      if (c < chunks) {
+        float o0[8], o1[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          o0[i] = go[b][i] * a0;
+          o1[i] = go[b][i] * a1;
+          dot0 += round_to<kF32>(go[b][i] * u[b][i]);
+          dot1 += round_to<kF32>(go[b][i] * v[b][i]);
+        }
+        store8_from_f32<kF32>(g_pub, t * dim + c * 8, o0);
+        store8_from_f32<kF32>(g_priv, t * dim + c * 8, o1);
+      }
+    }
+  }
+  dot0 = wave_sum(dot0);
+  dot1 = wave_sum(dot1);
+  if (lane == 0) {
+    if constexpr (kF32) {
+      reinterpret_cast<float*>(g_alpha)[2 * t] = dot0;
+      reinterpret_cast<float*>(g_alpha)[2 * t + 1] = dot1;
+    } else {
+      reinterpret_cast<uint32_t*>(g_alpha)[t] = pack_bf16x2(dot0, dot1);
+    }
+  }
+}
+
 // Zero-fill of the padded rows that hold no assignment, for the source-major
 // kernels below: wavefront w looks at rows 64w .. 64w+63 (one per lane) and the
 // whole wavefront then clears each invalid one.
@@ -520,5 +622,41 @@ extern "C" int nestor_hip_combine_rows_bwd(const void* grad_out, int32_t go_dtyp
     hipLaunchKernelGGL(combine_bwd_kernel<false>, dim3(row_blocks(rows_pad)),
                        dim3(kRowBlock), 0, s, grad_out, y, pad_src_row, pad_valid,
                        valid_dtype, weights, w_dtype, gy, grad_w, rows_pad, group, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_path_mix_fwd(const void* pub, const void* priv, const void* alpha,
+                                       void* out, int32_t dtype, int64_t num_tokens,
+                                       int64_t dim, void* stream) {
+  if (!dtype_ok(dtype) || dim <= 0 || dim % 8 != 0 || num_tokens < 0) return NESTOR_HIP_EINVAL;
+  if (num_tokens == 0) return NESTOR_HIP_OK;
+  if (!pub || !priv || !alpha || !out) return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(path_mix_fwd_kernel<true>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),
+                       0, s, pub, priv, alpha, out, num_tokens, dim);
+  else
+    hipLaunchKernelGGL(path_mix_fwd_kernel<false>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),
+                       0, s, pub, priv, alpha, out, num_tokens, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_path_mix_bwd(const void* grad_out, const void* pub, const void* priv,
+                                       const void* alpha, void* grad_pub, void* grad_priv,
+                                       void* grad_alpha, int32_t dtype, int64_t num_tokens,
+                                       int64_t dim, void* stream) {
+  if (!dtype_ok(dtype) || dim <= 0 || dim % 8 != 0 || num_tokens < 0) return NESTOR_HIP_EINVAL;
+  if (num_tokens == 0) return NESTOR_HIP_OK;
+  if (!grad_out || !pub || !priv || !alpha || !grad_pub || !grad_priv || !grad_alpha)
+    return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(path_mix_bwd_kernel<true>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),
+                       0, s, grad_out, pub, priv, alpha, grad_pub, grad_priv, grad_alpha,
+                       num_tokens, dim);
+  else
+    hipLaunchKernelGGL(path_mix_bwd_kernel<false>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),
+                       0, s, grad_out, pub, priv, alpha, grad_pub, grad_priv, grad_alpha,
+                       num_tokens, dim);
   return launch_status();
 }

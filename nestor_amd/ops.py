@@ -754,3 +754,76 @@ def _(scores, choice_bias, mask, top_k, gate_mode):
     n, c = scores.shape
     return [scores.new_empty(n, c, dtype=torch.float32),
             scores.new_empty(n, top_k, dtype=torch.long), torch.empty_like(scores)]
+
+
+# --------------------------------------------------------------------------
+# Path mix of the pool's summed layout
+# --------------------------------------------------------------------------
+def _mix_operands(alpha: Tensor, *tensors: Tensor) -> tuple[Tensor, ...]:
+    dtype = tensors[0].dtype
+    if any(t.dtype != dtype for t in tensors) or alpha.dtype != dtype:
+        raise TypeError("path mix operands must share one dtype")
+    if alpha.shape[-1] != 2 or alpha.numel() * tensors[0].shape[-1] != 2 * tensors[0].numel():
+        raise ValueError("alpha must be [..., 2] over the leading axes of the updates")
+    return tuple(t.contiguous() for t in (alpha, *tensors))
+
+
+@torch.library.custom_op(f"{_NS}::path_mix_fwd", mutates_args=(), device_types="cuda")
+def path_mix_fwd(public_update: Tensor, private_update: Tensor, alpha: Tensor) -> Tensor:
+    alpha, pub, priv = _mix_operands(alpha, public_update, private_update)
+    dim = pub.shape[-1]
+    out = torch.empty_like(pub)
+    _lib.call("nestor_hip_path_mix_fwd", _ptr(pub), _ptr(priv), _ptr(alpha), _ptr(out),
+              _code(pub.dtype), pub.numel() // dim, dim, _stream(pub))
+    return out
+
+
+@path_mix_fwd.register_fake
+def _(public_update, private_update, alpha):
+    return torch.empty_like(public_update)
+
+
+@torch.library.custom_op(f"{_NS}::path_mix_bwd", mutates_args=(), device_types="cuda")
+def path_mix_bwd(grad_out: Tensor, public_update: Tensor, private_update: Tensor,
+                 alpha: Tensor) -> list[Tensor]:
+    alpha, g, pub, priv = _mix_operands(alpha, grad_out, public_update, private_update)
+    dim = pub.shape[-1]
+    g_pub = torch.empty_like(pub)
+    g_priv = torch.empty_like(pub)
+    g_alpha = torch.empty_like(alpha)
+    _lib.call("nestor_hip_path_mix_bwd", _ptr(g), _ptr(pub), _ptr(priv), _ptr(alpha),
+              _ptr(g_pub), _ptr(g_priv), _ptr(g_alpha), _code(pub.dtype), pub.numel() // dim,
+              dim, _stream(pub))
+    return [g_pub, g_priv, g_alpha]
+
+
+@path_mix_bwd.register_fake
+def _(grad_out, public_update, private_update, alpha):
+    return [torch.empty_like(public_update), torch.empty_like(public_update),
+            torch.empty_like(alpha)]
+
+
+@torch.library.custom_op(f"{_NS}::path_mix", mutates_args=(), device_types="cuda")
+def path_mix_op(public_update: Tensor, private_update: Tensor, alpha: Tensor) -> Tensor:
+    """``alpha[..., 0:1] * public_update + alpha[..., 1:2] * private_update`` with the
+    eager expression's roundings, one launch (and one for all three gradients)."""
+
+    return path_mix_fwd(public_update, private_update, alpha)
+
+
+@path_mix_op.register_fake
+def _(public_update, private_update, alpha):
+    return torch.empty_like(public_update)
+
+
+def _path_mix_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs)
+
+
+def _path_mix_backward(ctx, grad_out):
+    pub, priv, alpha = ctx.saved_tensors
+    g_pub, g_priv, g_alpha = path_mix_bwd(grad_out.contiguous(), pub, priv, alpha)
+    return g_pub, g_priv, g_alpha
+
+
+path_mix_op.register_autograd(_path_mix_backward, setup_context=_path_mix_setup)

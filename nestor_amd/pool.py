@@ -19,7 +19,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from nestor_amd import flags
+from nestor_amd import flags, ops
 from nestor_amd.bank import Linear2, StackedBanksMixin, SwigluExpert
 from nestor_amd.grouped import grouped_expert_combine
 from nestor_amd.router import Router, RouterOutput, check_batchable, route_private_batched
@@ -307,8 +307,8 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
         if public_update is None:
             return private_update.to(x.dtype), pub_out, priv_outs
         alpha = self._path_weights(x)
-        update = alpha[..., 0:1] * public_update + alpha[..., 1:2] * private_update
-        return update.to(x.dtype), pub_out, priv_outs
+        update = ops.path_mix_op(public_update, private_update, alpha)
+        return update, pub_out, priv_outs
 
     def forward_per_slot(self, x: Tensor, valid_token_mask: Tensor, group_gates: Tensor,
                          group_active_mask: Tensor, slot_groups: Tensor, router_noise=None):

@@ -1,4 +1,4 @@
-"""Row-kernel oracles: dispatch gather, SwiGLU, cat+cast, weighted combine.
+"""Row-kernel oracles: dispatch gather, SwiGLU, cat+cast, weighted combine, path mix.
 
 Each forward is the eager chain the reference's fused kernels are held to; each
 backward states the reference's backward formula with its rounding points.
@@ -96,3 +96,20 @@ def combine_rows_bwd(
     gw = torch.zeros(weights.shape[0], dtype=torch.float32, device=y_pad.device)
     gw[src[valid]] = dots[valid]
     return gy, gw
+
+
+def path_mix(public_update: Tensor, private_update: Tensor, alpha: Tensor) -> Tensor:
+    """``alpha[..., 0:1] * public + alpha[..., 1:2] * private`` in the operands' dtype:
+    every product and the sum are rounded to it
+    (nestor/backbones/expert_pools.py:1110-1113)."""
+
+    return alpha[..., 0:1] * public_update + alpha[..., 1:2] * private_update
+
+
+def path_mix_bwd(grad_out: Tensor, public_update: Tensor, private_update: Tensor,
+                 alpha: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+    """What autograd derives from :func:`path_mix`: ``(g_public, g_private, g_alpha)``."""
+
+    leaves = [t.detach().clone().requires_grad_(True) for t in (public_update, private_update, alpha)]
+    path_mix(*leaves).backward(grad_out)
+    return leaves[0].grad, leaves[1].grad, leaves[2].grad

@@ -152,6 +152,32 @@ def test_source_major_and_row_major_kernels_agree(cuda, capacity):
         assert (plan.row_kept == 0).any()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(3, 50, 40), (1, 1, 8), (2, 300, 2048), (1, 257, 520)])
+def test_path_mix_fwd_bwd(cuda, dtype, shape):
+    """Values and input gradients are single rounded operations: exact.  The two
+    path-weight gradients are sums over the feature axis: within rounding."""
+
+    from nestor_amd import ops
+
+    b, s, d = shape
+    pub = torch.randn(b, s, d, generator=gen(1)).to(dtype)
+    priv = torch.randn(b, s, d, generator=gen(2)).to(dtype)
+    alpha = torch.softmax(torch.randn(b, s, 2, generator=gen(3)), -1).to(dtype)
+    go = torch.randn(b, s, d, generator=gen(4)).to(dtype)
+    want = orows.path_mix(pub, priv, alpha)
+    w_pub, w_priv, w_alpha = orows.path_mix_bwd(go, pub, priv, alpha)
+    leaves = [t.to(cuda).requires_grad_(True) for t in (pub, priv, alpha)]
+    out = ops.path_mix_op(*leaves)
+    assert out.dtype == dtype and out.shape == want.shape
+    assert torch.equal(out.cpu(), want)
+    out.backward(go.to(cuda))
+    assert torch.equal(leaves[0].grad.cpu(), w_pub)
+    assert torch.equal(leaves[1].grad.cpu(), w_priv)
+    tol = dict(rtol=2 ** -6, atol=0.05 * d ** 0.5) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4 * d ** 0.5)
+    torch.testing.assert_close(leaves[2].grad.cpu().float(), w_alpha.float(), **tol)
+
+
 def test_identity_round_trip(cuda):
     """combine(dispatch(x)) with unit weights sums each token's ``slots`` copies."""
 

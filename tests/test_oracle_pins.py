@@ -159,6 +159,28 @@ def test_combine_rows_loop_and_backward():
     assert (gy[plan.pad_valid == 0] == 0).all()
 
 
+def test_path_mix_loop_and_backward():
+    """Element loop with hand-placed roundings, then fp64 autograd of the definition."""
+
+    pub = torch.randn(7, 16, generator=gen(1)).bfloat16()
+    priv = torch.randn(7, 16, generator=gen(2)).bfloat16()
+    alpha = torch.softmax(torch.randn(7, 2, generator=gen(3)), -1).bfloat16()
+    out = orows.path_mix(pub, priv, alpha)
+    assert out.dtype == torch.bfloat16
+    for t in range(7):
+        for i in range(16):
+            a = (alpha[t, 0].float() * pub[t, i].float()).bfloat16().float()
+            b = (alpha[t, 1].float() * priv[t, i].float()).bfloat16().float()
+            assert out[t, i] == (a + b).bfloat16()
+    go = torch.randn(7, 16, generator=gen(4)).bfloat16()
+    g_pub, g_priv, g_alpha = orows.path_mix_bwd(go, pub, priv, alpha)
+    leaves = [t.double().requires_grad_(True) for t in (pub, priv, alpha)]
+    (leaves[2][:, 0:1] * leaves[0] + leaves[2][:, 1:2] * leaves[1]).backward(go.double())
+    for got, leaf in zip((g_pub, g_priv, g_alpha), leaves):
+        torch.testing.assert_close(got.double(), leaf.grad, rtol=2 ** -6, atol=2e-2)
+    assert not torch.equal(g_alpha[:, 0], g_alpha[:, 1])
+
+
 def test_segment_mm_and_bank_routes_agree():
     """grouped (padded) path == per-expert dense evaluation == sparse loop ==
     per-token loop, in fp32 where only summation order differs
