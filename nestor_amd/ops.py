@@ -827,3 +827,83 @@ def _path_mix_backward(ctx, grad_out):
 
 
 path_mix_op.register_autograd(_path_mix_backward, setup_context=_path_mix_setup)
+
+
+# --------------------------------------------------------------------------
+# Skinny score heads (router / path gate linear maps)
+# --------------------------------------------------------------------------
+@torch.library.custom_op(f"{_NS}::score_heads", mutates_args=(), device_types="cuda")
+def score_heads_op(x: Tensor, weight: Tensor, bias: Tensor | None) -> Tensor:
+    """``x [T, d] @ weight[C, d]^T (+ bias)`` in bf16, ``C`` a multiple of 8.
+
+    The forward is a library GEMM.  The input gradient ``g [T, C] @ weight`` has a
+    contraction of only ``C`` (tens to a few hundred) against ``T x d`` outputs: it is
+    a write-bound pass over the activations, and runs on the grouped GEMM kernel
+    with the whole batch as one bank."""
+
+    x = _bf16(x, "x")
+    weight = _bf16(weight, "weight")
+    if bias is None:
+        return x @ weight.t()
+    return torch.addmm(_bf16(bias, "bias"), x, weight.t())
+
+
+@score_heads_op.register_fake
+def _(x, weight, bias):
+    return x.new_empty(x.shape[0], weight.shape[0])
+
+
+_ONE_BANK_TABLES: dict[tuple[int, torch.device], Tensor] = {}
+
+
+def _one_bank_table(rows: int, device: torch.device) -> Tensor:
+    """Tile table of a single bank that owns rows ``0 .. rows``: a function of the row
+    count alone, built once per (count, device)."""
+
+    key = (rows, device)
+    table = _ONE_BANK_TABLES.get(key)
+    if table is None:
+        offs = torch.full((1,), rows, dtype=torch.int32, device=device)
+        table = tile_schedule(offs, rows)
+        if type(table) is Tensor:  # not while a compiler traces with stand-in tensors
+            _ONE_BANK_TABLES[key] = table
+    return table
+
+
+def _skinny_weight_grad(grad: Tensor, x: Tensor) -> Tensor:
+    """``grad [T, C]^T @ x [T, d]``: few outputs, a contraction over every row.  As
+    one GEMM it has ``C*d`` / tile-size workgroups (a few dozen) for the whole
+    device; split over row chunks it is a batched GEMM that fills the device, and
+    the chunk results (bf16) are summed in fp32."""
+
+    rows = x.shape[0]
+    chunks = 32
+    while chunks > 1 and (rows % chunks or rows // chunks < 512):
+        chunks //= 2
+    if chunks == 1:
+        return grad.t() @ x
+    parts = torch.bmm(grad.view(chunks, rows // chunks, -1).transpose(1, 2),
+                      x.view(chunks, rows // chunks, -1))
+    return parts.sum(0)
+
+
+def _score_heads_setup(ctx, inputs, output):
+    x, weight, bias = inputs
+    ctx.save_for_backward(x, weight)
+    ctx.has_bias = bias is not None
+
+
+def _score_heads_backward(ctx, grad):
+    x, weight = ctx.saved_tensors
+    grad = grad.contiguous()
+    gx = gw = gb = None
+    if ctx.needs_input_grad[0]:
+        gx = grouped_gemm_nn(grad, weight.unsqueeze(0), _one_bank_table(x.shape[0], x.device))
+    if ctx.needs_input_grad[1]:
+        gw = _skinny_weight_grad(grad, x)
+    if ctx.has_bias and ctx.needs_input_grad[2]:
+        gb = grad.sum(0)
+    return gx, gw, gb
+
+
+score_heads_op.register_autograd(_score_heads_backward, setup_context=_score_heads_setup)

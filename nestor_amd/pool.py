@@ -22,7 +22,9 @@ from torch import Tensor, nn
 from nestor_amd import flags, ops
 from nestor_amd.bank import Linear2, StackedBanksMixin, SwigluExpert
 from nestor_amd.grouped import grouped_expert_combine
-from nestor_amd.router import Router, RouterOutput, check_batchable, route_private_batched
+from nestor_amd.router import (
+    Router, RouterOutput, check_batchable, route_private_batched, score_linear,
+)
 
 
 def round_to_multiple_of_8(value: float) -> int:
@@ -230,7 +232,7 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
                 l.bias if l.bias is not None else l.weight.new_zeros(l.weight.shape[0])
                 for l in layers
             ])
-        out = F.linear(x.reshape(-1, self.dim), weight, bias)
+        out = score_linear(x.reshape(-1, self.dim), weight, bias)
         n_pub = layers[0].weight.shape[0]
         n_priv = sum(l.weight.shape[0] for l in layers[1:-1])
         return (out[:, :n_pub].reshape(*x.shape[:-1], n_pub), out[:, n_pub:n_pub + n_priv],

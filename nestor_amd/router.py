@@ -34,6 +34,31 @@ class RouterOutput(NamedTuple):
     valid_token_mask: Tensor
 
 
+def score_linear(x: Tensor, weight: Tensor, bias: Tensor | None) -> Tensor:
+    """``F.linear`` for a skinny score head over rows ``x [T, d]``.  When the GEMM runs
+    in bf16 on the GPU and ``x`` needs a gradient, the input gradient goes through the
+    grouped GEMM kernel (``ops.score_heads_op``); the head count is padded with zero
+    rows to a multiple of 32 for it.  Values are those of ``F.linear``."""
+
+    bf16 = torch.bfloat16
+    if x.is_cuda and torch.is_autocast_enabled("cuda"):
+        on_bf16 = torch.get_autocast_dtype("cuda") == bf16
+    else:
+        on_bf16 = x.dtype == bf16 and weight.dtype == bf16
+    if not (x.is_cuda and on_bf16 and x.dim() == 2 and torch.is_grad_enabled() and x.requires_grad):
+        return F.linear(x, weight, bias)
+    heads = weight.shape[0]
+    pad = -heads % 32
+    w = weight.to(bf16)
+    b = None if bias is None else bias.to(bf16)
+    if pad:
+        w = torch.cat([w, w.new_zeros(pad, w.shape[1])])
+        b = None if b is None else torch.cat([b, b.new_zeros(pad)])
+    with torch.autocast("cuda", enabled=False):
+        out = ops.score_heads_op(x.to(bf16), w, b)
+    return out[:, :heads] if pad else out
+
+
 class ScoreMLP(nn.Module):
     """Score head: ``Linear`` layers with an activation between them (none after
     the last); ``hidden_dims=[]`` is the single linear map every registered arm uses."""
@@ -56,7 +81,11 @@ class ScoreMLP(nn.Module):
     def forward(self, x: Tensor) -> Tensor:
         for layer in self.layers[:-1]:
             x = self._activation_fn(layer(x))
-        return self.layers[-1](x)
+        last = self.layers[-1]
+        if x.dim() >= 2 and len(self.layers) == 1:
+            flat = score_linear(x.reshape(-1, x.shape[-1]), last.weight, last.bias)
+            return flat.reshape(*x.shape[:-1], flat.shape[-1])
+        return last(x)
 
 
 def _softmax_dtype(scores: Tensor) -> torch.dtype:
@@ -160,7 +189,7 @@ def batched_mlp(x: Tensor, mlps: list[ScoreMLP]) -> Tensor:
         torch.stack([m.layers[0].bias for m in mlps]).reshape(-1)
         if mlps[0].layers[0].bias is not None else None
     )
-    hidden = F.linear(x, w0.reshape(heads * w0.shape[1], w0.shape[2]), b0)
+    hidden = score_linear(x, w0.reshape(heads * w0.shape[1], w0.shape[2]), b0)
     hidden = hidden.view(x.shape[0], heads, w0.shape[1])
     for index in range(1, len(mlps[0].layers)):
         hidden = mlps[0]._activation_fn(hidden)

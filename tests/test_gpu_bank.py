@@ -183,3 +183,38 @@ def test_full_size_pool_step_vs_gold_on_gpu(cuda, workload, seeds):
                 assert rel_l2(got, want.grad) < 1.5e-2, (workload, seed, n)
         del gold_params, total, xs, t, pool, captured
         torch.cuda.empty_cache()
+
+
+def test_bank_call_traces_under_torch_compile(cuda):
+    """The custom ops carry shape-only kernels and registered gradients, so a bank
+    call compiles (``aot_eager``: traced forward and backward graphs, run op by op)
+    and gives the eager path's bits."""
+
+    from nestor_amd import StackedExpertBank, grouped_expert_combine
+
+    tokens, d, h, banks, slots, group = 512, 256, 512, 8, 2, 2
+    ids, weights = routing(3, tokens, slots, banks)
+    x = torch.randn(tokens, d, generator=gen(0)).bfloat16()
+    w3 = bank_weights(1, banks, d, h, 0.05, torch.bfloat16)
+    go = torch.randn(tokens, 1, d, generator=gen(2)).bfloat16().to(cuda)
+    bank = StackedExpertBank.from_tensors(*[t.clone() for t in w3]).to(cuda)
+    dev_ids = ids.to(cuda)
+
+    def call(tx, tw):
+        return grouped_expert_combine(
+            tx, bank.expert_views(), dev_ids, tw, group, fused_gate=True, stacked=bank,
+            triton_index=True, triton_fused=True,
+        )
+
+    results = []
+    for fn in (call, torch.compile(call, backend="aot_eager")):
+        for t in (bank.w_up, bank.w_gate, bank.w_down):
+            t.grad = None
+        tx = x.to(cuda).requires_grad_(True)
+        tw = weights.bfloat16().to(cuda).requires_grad_(True)
+        out = fn(tx, tw)
+        out.backward(go)
+        results.append([out.detach(), tx.grad, tw.grad, bank.w_up.grad, bank.w_gate.grad,
+                        bank.w_down.grad])
+    for eager, compiled in zip(*results):
+        assert torch.equal(eager, compiled)

@@ -100,3 +100,35 @@ def test_pool_routing_matches_oracle_slots(cuda):
     opub = orouter.route(pub.scores.cpu()[0], torch.zeros(w.public), 1, "renorm", valid.cpu()[0])
     assert torch.equal(pub_ids.cpu(), opub.topk_indices)
     assert torch.equal(pub_w.cpu().float(), torch.ones(w.tokens, 1))
+
+
+@pytest.mark.parametrize("tokens,dim,heads,bias", [
+    (300, 64, 10, True), (1000, 512, 146, False), (129, 1024, 32, True), (4096, 2048, 160, False),
+])
+def test_score_linear_matches_linear(cuda, tokens, dim, heads, bias):
+    """Skinny score heads: values are the library GEMM's; the input gradient comes
+    from the grouped GEMM kernel (whole batch as one bank, head count zero-padded
+    to a multiple of 32) and is held to the fp32 product of the same bf16 operands."""
+
+    from nestor_amd.router import score_linear
+    from tests.helpers import rel_l2
+
+    x = torch.randn(tokens, dim, generator=gen(1)).bfloat16()
+    w = (torch.randn(heads, dim, generator=gen(2)) / dim ** 0.5).bfloat16()
+    b = torch.randn(heads, generator=gen(3)).bfloat16() if bias else None
+    g = torch.randn(tokens, heads, generator=gen(4)).bfloat16()
+    tx = x.to(cuda).requires_grad_(True)
+    tw = w.to(cuda).requires_grad_(True)
+    tb = b.to(cuda).requires_grad_(True) if bias else None
+    out = score_linear(tx, tw, tb)
+    ref = torch.nn.functional.linear(x.float(), w.float(), None if b is None else b.float())
+    assert out.shape == ref.shape and out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=2 ** -6, atol=2e-2)
+    out.backward(g.to(cuda))
+    assert rel_l2(tx.grad, g.float() @ w.float()) < 4e-3
+    assert rel_l2(tw.grad, g.float().t() @ x.float()) < 4e-3
+    if bias:
+        assert rel_l2(tb.grad, g.float().sum(0)) < 4e-3
+    # without a gradient on the rows the library path runs and gives the same values
+    plain = score_linear(x.to(cuda), tw, tb)
+    assert torch.equal(plain, out)
