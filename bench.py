@@ -293,7 +293,8 @@ def main() -> None:
     if dom:
         roofline = {
             "bound": "mfma",
-            "kernel": "grouped_gemm_kernel<kNNUpGate> (private bank up|gate + SwiGLU)",
+            "kernel": "grouped_gemm_dma_kernel<DmaCfg<128,512,32,1,4,3>, kNNUpGate> "
+                      "(private bank up|gate + SwiGLU)",
             "achieved": dom["tflops"],
             "peak": BF16_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
