@@ -123,6 +123,22 @@ def kernel_breakdown(w, tensors, iters: int = 5) -> dict:
     ms = _event_ms(lambda: ops.dispatch_rows_bwd(gx_pad, plan.row_dest, T, slots, torch.bfloat16), iters)
     report("dispatch_bwd", ms, bytes_=rows * d * 2 + T * d * 2)
     del o
+
+    # pool epilogues: the summed layout's path mix and the column layout's scatter
+    alpha = torch.softmax(torch.randn(T, 2, generator=g, device=dev), -1).to(torch.bfloat16)
+    pub, priv = x, gx_pad[:T]
+    ms = _event_ms(lambda: ops.path_mix_fwd(pub, priv, alpha), iters)
+    report("path_mix_fwd", ms, bytes_=3 * T * d * 2)
+    ms = _event_ms(lambda: ops.path_mix_bwd(go, pub, priv, alpha), iters)
+    report("path_mix_bwd", ms, bytes_=5 * T * d * 2)
+    k_a = w.k_columns
+    per_slot = gx_pad[: T * k_a].view(T, k_a, d)
+    columns = torch.rand(T, w.columns, generator=g, device=dev).topk(k_a, -1).indices
+    ms = _event_ms(lambda: ops.path_scale_fwd(per_slot, alpha, 1, columns, w.columns), iters)
+    report("column_scatter_fwd", ms, bytes_=T * k_a * d * 2 + T * w.columns * d * 2)
+    g_cols = ops.path_scale_fwd(per_slot, alpha, 1, columns, w.columns)
+    ms = _event_ms(lambda: ops.path_scale_bwd(g_cols, per_slot, alpha, 1, columns), iters)
+    report("column_scatter_bwd", ms, bytes_=3 * T * k_a * d * 2)
     return out
 
 

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 3
+#define NESTOR_HIP_ABI_VERSION 4
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -278,6 +278,26 @@ int nestor_hip_path_mix_bwd(
     const void* grad_out, const void* public_update, const void* private_update,
     const void* alpha, void* grad_public, void* grad_private, void* grad_alpha,
     int32_t dtype, int64_t num_tokens, int64_t dim, void* stream);
+
+/* Split layouts of the pool (nestor/backbones/expert_pools.py:943-953 per slot,
+ * :1023-1041 per column): out[t,o,:] = alpha[t,which] * X[t,o,:] rounded to
+ * `dtype`, where X = in ([num_tokens, slots, dim]; dest == NULL, num_out ==
+ * slots) or in scattered onto num_out column streams by dest [num_tokens, slots]
+ * (the zeros(...).scatter_add(1, index, per_slot) of :758-761; streams no slot
+ * selects are zero).  dest entries must lie in [0, num_out).  slots <= 64. */
+int nestor_hip_path_scale_fwd(
+    const void* in, const void* alpha /* [num_tokens, 2] */, int32_t which,
+    const int64_t* dest /* nullable */, void* out /* [num_tokens, num_out, dim] */,
+    int32_t dtype, int64_t num_tokens, int32_t slots, int32_t num_out, int64_t dim,
+    void* stream);
+/* grad_in[t,s,:] = grad_out[t,o(s),:] * alpha[t,which] with o(s) = dest[t,s] (or s);
+ * grad_alpha[t] = sum over slots and features of grad_out[t,o(s),:] * in[t,s,:]
+ * (fp32): the gradient of alpha[t,which]. */
+int nestor_hip_path_scale_bwd(
+    const void* grad_out, const void* in, const void* alpha, int32_t which,
+    const int64_t* dest /* nullable */, void* grad_in, float* grad_alpha /* [num_tokens] */,
+    int32_t dtype, int64_t num_tokens, int32_t slots, int32_t num_out, int64_t dim,
+    void* stream);
 
 #ifdef __cplusplus
 }

@@ -405,6 +405,117 @@ __global__ __launch_bounds__(kRowBlock) void path_mix_bwd_kernel(
   }
 }
 
+// Split layouts of the pool: out[t,o,:] = alpha[t,which] * X[t,o,:] where X is the
+// input itself (dest == nullptr, num_out == slots) or its slots scattered onto
+// num_out column streams, X[t,o,:] = sum of in[t,s,:] over the slots with
+// dest[t,s] == o (slot order, each partial sum rounded as an eager scatter_add
+// in the tensor's dtype rounds it), zero for streams no slot selects.
+template <bool kF32>
+__global__ __launch_bounds__(kRowBlock) void path_scale_fwd_kernel(
+    const void* __restrict__ in, const void* __restrict__ alpha, int which,
+    const int64_t* __restrict__ dest, void* __restrict__ out, int64_t num_tokens, int slots,
+    int num_out, int64_t dim) {
+#pragma clang fp contract(off)
+  // With a scatter most output rows are zero fill: a wavefront takes kOutRows
+  // consecutive streams of one token so that it has enough stores to issue.
+  constexpr int kOutRows = 8;
+  const int groups = (num_out + kOutRows - 1) / kOutRows;
+  const int64_t w = wave_row();
+  if (w >= num_tokens * groups) return;
+  const int64_t t = w / groups;
+  const int o0 = static_cast<int>(w - t * groups) * kOutRows;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const int dt = kF32 ? NESTOR_HIP_F32 : NESTOR_HIP_BF16;
+  const float a = load_scalar(alpha, 2 * t + which, dt);
+  // lane s holds the stream of slot s (slots <= 64)
+  const int64_t mine = dest == nullptr ? lane : (lane < slots ? dest[t * slots + lane] : -1);
+  for (int o = o0; o < o0 + kOutRows && o < num_out; ++o) {
+    // slots that feed this output row, as a bit mask
+    const uint64_t feeds = __ballot(lane < slots && mine == o);
+    const int64_t row = t * num_out + o;
+    for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+      float acc[kBatch][8];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[b][i] = 0.0f;
+      for (uint64_t todo = feeds; todo != 0; todo &= todo - 1) {
+        const int s = __ffsll(static_cast<long long>(todo)) - 1;
+        const int64_t base = (t * slots + s) * dim;
+        float v[kBatch][8];
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b)
+          if (c0 + b * kWave < chunks) load8_as_f32<kF32>(in, base + (c0 + b * kWave) * 8, v[b]);
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b)
+          if (c0 + b * kWave < chunks)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[b][i] = round_to<kF32>(acc[b][i] + v[b][i]);
+      }
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        const int c = c0 + b * kWave;
+        if (c < chunks) {
+          float r[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) r[i] = a * acc[b][i];
+          store8_from_f32<kF32>(out, row * dim + c * 8, r);
+        }
+      }
+    }
+  }
+}
+
+// grad_in[t,s,:] = g[t,o(s),:] * alpha[t,which] (rounded);
+// grad_alpha[t] = sum_s sum_d round(g[t,o(s),:] * in[t,s,:]) in fp32, o(s) = dest[t,s]
+// or s.  One wavefront per token walks its slots in order.
+template <bool kF32>
+__global__ __launch_bounds__(kRowBlock) void path_scale_bwd_kernel(
+    const void* __restrict__ g, const void* __restrict__ in, const void* __restrict__ alpha,
+    int which, const int64_t* __restrict__ dest, void* __restrict__ g_in,
+    float* __restrict__ g_alpha, int64_t num_tokens, int slots, int num_out, int64_t dim) {
+#pragma clang fp contract(off)
+  const int64_t t = wave_row();
+  if (t >= num_tokens) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const int dt = kF32 ? NESTOR_HIP_F32 : NESTOR_HIP_BF16;
+  const float a = load_scalar(alpha, 2 * t + which, dt);
+  float dot = 0.0f;
+  for (int s = 0; s < slots; ++s) {
+    const int64_t o = dest == nullptr ? s : dest[t * slots + s];
+    const int64_t gbase = (t * num_out + o) * dim;
+    const int64_t ibase = (t * slots + s) * dim;
+    for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+      float go[kBatch][8], v[kBatch][8];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        const int c = c0 + b * kWave;
+        if (c < chunks) {
+          load8_as_f32<kF32>(g, gbase + c * 8, go[b]);
+          load8_as_f32<kF32>(in, ibase + c * 8, v[b]);
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        const int c = c0 + b * kWave;
+        if (c < chunks) {
+          float r[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            r[i] = go[b][i] * a;
+            dot += round_to<kF32>(go[b][i] * v[b][i]);
+          }
+          store8_from_f32<kF32>(g_in, ibase + c * 8, r);
+        }
+      }
+    }
+  }
+  dot = wave_sum(dot);
+  if (lane == 0) g_alpha[t] = dot;
+}
+
 // Zero-fill of the padded rows that hold no assignment, for the source-major
 // kernels below: wavefront w looks at rows 64w .. 64w+63 (one per lane) and the
 // whole wavefront then clears each invalid one.
@@ -658,5 +769,49 @@ extern "C" int nestor_hip_path_mix_bwd(const void* grad_out, const void* pub, co
     hipLaunchKernelGGL(path_mix_bwd_kernel<false>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),
                        0, s, grad_out, pub, priv, alpha, grad_pub, grad_priv, grad_alpha,
                        num_tokens, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_path_scale_fwd(const void* in, const void* alpha, int32_t which,
+                                         const int64_t* dest, void* out, int32_t dtype,
+                                         int64_t num_tokens, int32_t slots, int32_t num_out,
+                                         int64_t dim, void* stream) {
+  if (!dtype_ok(dtype) || dim <= 0 || dim % 8 != 0 || num_tokens < 0 || slots <= 0 ||
+      slots > 64 || num_out <= 0 || (which != 0 && which != 1) ||
+      (dest == nullptr && num_out != slots))
+    return NESTOR_HIP_EINVAL;
+  if (num_tokens == 0) return NESTOR_HIP_OK;
+  if (!in || !alpha || !out) return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t rows = num_tokens * ((num_out + 7) / 8);  // wavefronts: 8 streams each
+  if (dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(path_scale_fwd_kernel<true>, dim3(row_blocks(rows)), dim3(kRowBlock), 0, s,
+                       in, alpha, which, dest, out, num_tokens, slots, num_out, dim);
+  else
+    hipLaunchKernelGGL(path_scale_fwd_kernel<false>, dim3(row_blocks(rows)), dim3(kRowBlock), 0, s,
+                       in, alpha, which, dest, out, num_tokens, slots, num_out, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_path_scale_bwd(const void* grad_out, const void* in, const void* alpha,
+                                         int32_t which, const int64_t* dest, void* grad_in,
+                                         float* grad_alpha, int32_t dtype, int64_t num_tokens,
+                                         int32_t slots, int32_t num_out, int64_t dim,
+                                         void* stream) {
+  if (!dtype_ok(dtype) || dim <= 0 || dim % 8 != 0 || num_tokens < 0 || slots <= 0 ||
+      slots > 64 || num_out <= 0 || (which != 0 && which != 1) ||
+      (dest == nullptr && num_out != slots))
+    return NESTOR_HIP_EINVAL;
+  if (num_tokens == 0) return NESTOR_HIP_OK;
+  if (!grad_out || !in || !alpha || !grad_in || !grad_alpha) return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(path_scale_bwd_kernel<true>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),
+                       0, s, grad_out, in, alpha, which, dest, grad_in, grad_alpha, num_tokens,
+                       slots, num_out, dim);
+  else
+    hipLaunchKernelGGL(path_scale_bwd_kernel<false>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),
+                       0, s, grad_out, in, alpha, which, dest, grad_in, grad_alpha, num_tokens,
+                       slots, num_out, dim);
   return launch_status();
 }

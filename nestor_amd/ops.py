@@ -829,6 +829,80 @@ def _path_mix_backward(ctx, grad_out):
 path_mix_op.register_autograd(_path_mix_backward, setup_context=_path_mix_setup)
 
 
+@torch.library.custom_op(f"{_NS}::path_scale_fwd", mutates_args=(), device_types="cuda")
+def path_scale_fwd(inp: Tensor, alpha: Tensor, which: int, dest: Tensor | None,
+                   num_out: int) -> Tensor:
+    inp = inp.contiguous()
+    alpha = alpha.contiguous()
+    if alpha.dtype != inp.dtype:
+        raise TypeError("path scale operands must share one dtype")
+    slots, dim = inp.shape[-2], inp.shape[-1]
+    tokens = inp.numel() // (slots * dim)
+    d = None if dest is None else dest.contiguous()
+    out = torch.empty(*inp.shape[:-2], num_out, dim, dtype=inp.dtype, device=inp.device)
+    _lib.call("nestor_hip_path_scale_fwd", _ptr(inp), _ptr(alpha), which, _ptr(d), _ptr(out),
+              _code(inp.dtype), tokens, slots, num_out, dim, _stream(inp))
+    return out
+
+
+@path_scale_fwd.register_fake
+def _(inp, alpha, which, dest, num_out):
+    return inp.new_empty(*inp.shape[:-2], num_out, inp.shape[-1])
+
+
+@torch.library.custom_op(f"{_NS}::path_scale_bwd", mutates_args=(), device_types="cuda")
+def path_scale_bwd(grad_out: Tensor, inp: Tensor, alpha: Tensor, which: int,
+                   dest: Tensor | None) -> list[Tensor]:
+    grad_out = grad_out.contiguous()
+    inp = inp.contiguous()
+    alpha = alpha.contiguous()
+    slots, dim = inp.shape[-2], inp.shape[-1]
+    tokens = inp.numel() // (slots * dim)
+    d = None if dest is None else dest.contiguous()
+    g_in = torch.empty_like(inp)
+    g_alpha = torch.empty(alpha.shape[:-1], dtype=torch.float32, device=inp.device)
+    _lib.call("nestor_hip_path_scale_bwd", _ptr(grad_out), _ptr(inp), _ptr(alpha), which, _ptr(d),
+              _ptr(g_in), _ptr(g_alpha), _code(inp.dtype), tokens, slots, grad_out.shape[-2], dim,
+              _stream(inp))
+    return [g_in, g_alpha]
+
+
+@path_scale_bwd.register_fake
+def _(grad_out, inp, alpha, which, dest):
+    return [torch.empty_like(inp), alpha.new_empty(alpha.shape[:-1], dtype=torch.float32)]
+
+
+@torch.library.custom_op(f"{_NS}::path_scale", mutates_args=(), device_types="cuda")
+def path_scale_op(inp: Tensor, alpha: Tensor, which: int, dest: Tensor | None,
+                  num_out: int) -> Tensor:
+    """``alpha[..., which] * X`` for ``inp [..., slots, d]``: ``X = inp`` or, with ``dest
+    [..., slots]``, ``zeros(..., num_out, d).scatter_add(-2, dest, inp)``."""
+
+    return path_scale_fwd(inp, alpha, which, dest, num_out)
+
+
+@path_scale_op.register_fake
+def _(inp, alpha, which, dest, num_out):
+    return inp.new_empty(*inp.shape[:-2], num_out, inp.shape[-1])
+
+
+def _path_scale_setup(ctx, inputs, output):
+    inp, alpha, which, dest, _num_out = inputs
+    ctx.save_for_backward(inp, alpha, dest)
+    ctx.which = which
+
+
+def _path_scale_backward(ctx, grad_out):
+    inp, alpha, dest = ctx.saved_tensors
+    g_in, g_col = path_scale_bwd(grad_out, inp, alpha, ctx.which, dest)
+    g_alpha = torch.zeros_like(alpha)
+    g_alpha[..., ctx.which] = g_col.to(alpha.dtype)
+    return g_in, g_alpha, None, None, None
+
+
+path_scale_op.register_autograd(_path_scale_backward, setup_context=_path_scale_setup)
+
+
 # --------------------------------------------------------------------------
 # Skinny score heads (router / path gate linear maps)
 # --------------------------------------------------------------------------

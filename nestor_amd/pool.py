@@ -336,18 +336,28 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
         )
         ids, weights, selected = self._private_slots(priv_outs, flat_gates, n, stacked=stacked)
         per_slot = self._private_per_slot(flat_x, ids, weights)
-        index = selected.unsqueeze(-1).expand(-1, -1, self.dim)
-        per_group = flat_x.new_zeros(n, self.num_groups, self.dim).scatter_add(1, index, per_slot)
-        per_group = per_group.view(x.shape[0], x.shape[1], self.num_groups, self.dim)
-        return self._gate_split(x, public_update, per_group, pub_out, priv_outs)
+        return self._gate_split(x, public_update, per_slot, pub_out, priv_outs, columns=selected)
 
-    def _gate_split(self, x, public_update, private_split, pub_out, priv_outs):
+    def _gate_split(self, x, public_update, per_slot, pub_out, priv_outs, columns=None):
+        """Outputs of the split layouts from the per-slot rows ``[n or B,S, k_a, d]``.
+        ``columns [n, k_a]`` scatters the slots onto the ``G`` column streams
+        (``zeros.scatter_add`` in the reference, expert_pools.py:758-761); the path
+        weights scale both parts.  One launch per part."""
+
+        lead = x.shape[:-1]
+        per_slot = per_slot.reshape(*lead, -1, self.dim)
+        width = per_slot.shape[-2] if columns is None else self.num_groups
+        dest = None if columns is None else columns.reshape(*lead, -1)
         if public_update is None:
-            return None, private_split.to(x.dtype), pub_out, priv_outs
+            if dest is None:
+                return None, per_slot.to(x.dtype), pub_out, priv_outs
+            ones = per_slot.new_ones(*lead, 2)  # a private-only pool has the constant weight 1
+            return None, ops.path_scale_op(per_slot, ones, 1, dest, width), pub_out, priv_outs
         alpha = self._path_weights(x)
         return (
-            (alpha[..., 0:1] * public_update).to(x.dtype),
-            (alpha[..., 1:2].unsqueeze(-1) * private_split).to(x.dtype),
+            ops.path_scale_op(public_update.reshape(*lead, 1, self.dim), alpha, 0, None, 1)
+            .reshape_as(x),
+            ops.path_scale_op(per_slot, alpha, 1, dest, width),
             pub_out,
             priv_outs,
         )

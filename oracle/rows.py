@@ -113,3 +113,26 @@ def path_mix_bwd(grad_out: Tensor, public_update: Tensor, private_update: Tensor
     leaves = [t.detach().clone().requires_grad_(True) for t in (public_update, private_update, alpha)]
     path_mix(*leaves).backward(grad_out)
     return leaves[0].grad, leaves[1].grad, leaves[2].grad
+
+
+def path_scale(inp: Tensor, alpha: Tensor, which: int, dest: Tensor | None = None,
+               num_out: int = 0) -> Tensor:
+    """Split layouts of the pool: ``alpha[..., which] * X`` with ``X = inp [..., slots, d]``
+    (per slot, nestor/backbones/expert_pools.py:943-953) or ``inp`` scattered onto
+    ``num_out`` column streams by ``dest [..., slots]``
+    (``zeros.scatter_add``, expert_pools.py:758-761, scaled at :1031-1041)."""
+
+    x = inp
+    if dest is not None:
+        index = dest.unsqueeze(-1).expand_as(inp)
+        x = inp.new_zeros(*inp.shape[:-2], num_out, inp.shape[-1]).scatter_add(-2, index, inp)
+    return alpha[..., which:which + 1].unsqueeze(-1) * x
+
+
+def path_scale_bwd(grad_out: Tensor, inp: Tensor, alpha: Tensor, which: int,
+                   dest: Tensor | None = None, num_out: int = 0) -> tuple[Tensor, Tensor]:
+    """What autograd derives from :func:`path_scale`: ``(g_inp, g_alpha [..., 2])``."""
+
+    leaves = [t.detach().clone().requires_grad_(True) for t in (inp, alpha)]
+    path_scale(leaves[0], leaves[1], which, dest, num_out).backward(grad_out)
+    return leaves[0].grad, leaves[1].grad

@@ -178,6 +178,38 @@ def test_path_mix_fwd_bwd(cuda, dtype, shape):
     torch.testing.assert_close(leaves[2].grad.cpu().float(), w_alpha.float(), **tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("tokens,slots,cols,d", [(50, 2, 8, 40), (1, 1, 1, 8), (300, 2, 32, 2048),
+                                                 (257, 3, 0, 520), (64, 4, 4, 64)])
+def test_path_scale_fwd_bwd(cuda, dtype, tokens, slots, cols, d):
+    """Per-slot scaling (``cols == 0``) and the scatter onto column streams: values and
+    the input gradient exact, the path-weight gradient within rounding of the sum."""
+
+    from nestor_amd import ops
+
+    inp = torch.randn(2, tokens, slots, d, generator=gen(1)).to(dtype)
+    alpha = torch.softmax(torch.randn(2, tokens, 2, generator=gen(2)), -1).to(dtype)
+    dest = None
+    if cols:
+        dest = torch.stack([torch.randperm(cols, generator=gen(10 + t))[:slots]
+                            for t in range(2 * tokens)]).view(2, tokens, slots)
+    width = cols or slots
+    go = torch.randn(2, tokens, width, d, generator=gen(3)).to(dtype)
+    for which in (0, 1):
+        want = orows.path_scale(inp, alpha, which, dest, cols)
+        w_in, w_alpha = orows.path_scale_bwd(go, inp, alpha, which, dest, cols)
+        t_in = inp.to(cuda).requires_grad_(True)
+        t_alpha = alpha.to(cuda).requires_grad_(True)
+        out = ops.path_scale_op(t_in, t_alpha, which, None if dest is None else dest.to(cuda), width)
+        assert out.dtype == dtype and torch.equal(out.cpu(), want)
+        out.backward(go.to(cuda))
+        assert torch.equal(t_in.grad.cpu(), w_in)
+        scale = (slots * d) ** 0.5
+        tol = dict(rtol=2 ** -6, atol=0.05 * scale) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4 * scale)
+        torch.testing.assert_close(t_alpha.grad.cpu().float(), w_alpha.float(), **tol)
+        assert (t_alpha.grad[..., 1 - which] == 0).all()
+
+
 def test_identity_round_trip(cuda):
     """combine(dispatch(x)) with unit weights sums each token's ``slots`` copies."""
 

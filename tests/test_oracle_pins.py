@@ -181,6 +181,34 @@ def test_path_mix_loop_and_backward():
     assert not torch.equal(g_alpha[:, 0], g_alpha[:, 1])
 
 
+def test_path_scale_loop():
+    """Column scatter + path weight against an element loop (distinct columns per token,
+    as top-k selection gives them)."""
+
+    tokens, slots, cols, d = 9, 2, 5, 8
+    inp = torch.randn(tokens, slots, d, generator=gen(1)).bfloat16()
+    alpha = torch.softmax(torch.randn(tokens, 2, generator=gen(2)), -1).bfloat16()
+    dest = torch.stack([torch.randperm(cols, generator=gen(10 + t))[:slots] for t in range(tokens)])
+    out = orows.path_scale(inp, alpha, 1, dest, cols)
+    assert out.shape == (tokens, cols, d)
+    for t in range(tokens):
+        for o in range(cols):
+            hit = [s for s in range(slots) if dest[t, s] == o]
+            for i in range(d):
+                want = (alpha[t, 1].float() * inp[t, hit[0], i].float()).bfloat16() if hit else 0.0
+                assert out[t, o, i] == want
+    plain = orows.path_scale(inp, alpha, 0)
+    assert torch.equal(plain, alpha[:, 0:1, None] * inp)
+    go = torch.randn(tokens, cols, d, generator=gen(3)).bfloat16()
+    g_in, g_alpha = orows.path_scale_bwd(go, inp, alpha, 1, dest, cols)
+    assert (g_alpha[:, 0] == 0).all()
+    for t in range(tokens):
+        picked = go[t, dest[t]].float()
+        torch.testing.assert_close(g_in[t].float(), picked * alpha[t, 1].float(), rtol=2 ** -7, atol=1e-6)
+        torch.testing.assert_close(g_alpha[t, 1].float(), (picked * inp[t].float()).sum(),
+                                   rtol=2 ** -6, atol=5e-2)
+
+
 def test_segment_mm_and_bank_routes_agree():
     """grouped (padded) path == per-expert dense evaluation == sparse loop ==
     per-token loop, in fp32 where only summation order differs
