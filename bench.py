@@ -124,6 +124,10 @@ def kernel_breakdown(w, tensors, iters: int = 5) -> dict:
     report("dispatch_bwd", ms, bytes_=rows * d * 2 + T * d * 2)
     del o
 
+    # biased banks: the bias gradient as a segmented column sum over the padded rows
+    ms = _event_ms(lambda: ops.segment_colsum(gh, None, plan.padded_starts, plan.counts), iters)
+    report("bias_grad_colsum", ms, bytes_=rows * h * 2)
+
     # pool epilogues: the summed layout's path mix and the column layout's scatter
     alpha = torch.softmax(torch.randn(T, 2, generator=g, device=dev), -1).to(torch.bfloat16)
     pub, priv = x, gx_pad[:T]

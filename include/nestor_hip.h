@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 4
+#define NESTOR_HIP_ABI_VERSION 5
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -298,6 +298,31 @@ int nestor_hip_path_scale_bwd(
     const int64_t* dest /* nullable */, void* grad_in, float* grad_alpha /* [num_tokens] */,
     int32_t dtype, int64_t num_tokens, int32_t slots, int32_t num_out, int64_t dim,
     void* stream);
+
+/* ------------------------------------------------------------------------
+ * Biased banks (the reference's native MoE baselines:
+ * nestor/backbones/grouped_mm.py:159-177 _IndexedBias, :426-437 up bias on the
+ * padded rows, :541-554 down bias on the routed rows).
+ * out[r,:] = bf16(rows[r,:] + bias[index[r],:]) where valid[r] != 0 (every row
+ * when valid == NULL), rows[r,:] elsewhere.  rows/out bf16 [n_rows, dim], bias
+ * bf16 [E, dim].
+ * ---------------------------------------------------------------------- */
+int nestor_hip_bias_rows_fwd(
+    const void* rows, const void* bias, const int64_t* index,
+    const void* valid /* nullable */, int32_t valid_dtype, void* out,
+    int64_t n_rows, int64_t dim, void* stream);
+/* The bias gradient, the reference's one-hot GEMM (onehot[E,rows] @ grad_rows,
+ * :173-177) as a segmented column sum: out[e,:] = bf16( sum_{i < seg_count[e]}
+ * grad[row(e,i),:] ), row(e,i) = row_index[seg_start[e]+i], or seg_start[e]+i
+ * when row_index == NULL (padded rows: seg_start = padded_starts; routed rows:
+ * row_index = the plan's stable order, seg_start = raw_starts).  fp32 sums in a
+ * fixed order, no atomics.  splits > 1 divides every segment over that many
+ * workgroups and needs partial [splits, E, dim] fp32. */
+int nestor_hip_segment_colsum(
+    const void* grad /* bf16 [*, dim] */, const int64_t* row_index /* nullable */,
+    const int64_t* seg_start, const int64_t* seg_count,
+    float* partial /* nullable when splits == 1 */, int32_t splits,
+    void* out /* bf16 [E, dim] */, int32_t num_banks, int64_t dim, void* stream);
 
 #ifdef __cplusplus
 }

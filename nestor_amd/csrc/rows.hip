@@ -516,6 +516,122 @@ __global__ __launch_bounds__(kRowBlock) void path_scale_bwd_kernel(
   if (lane == 0) g_alpha[t] = dot;
 }
 
+// Biased banks: out[r,:] = rows[r,:] + bias[index[r],:] (rounded to bf16) on rows
+// that hold an assignment, rows[r,:] unchanged elsewhere.
+__global__ __launch_bounds__(kRowBlock) void bias_rows_fwd_kernel(
+    const uint16_t* __restrict__ rows, const uint16_t* __restrict__ bias,
+    const int64_t* __restrict__ index, const void* __restrict__ valid, int valid_dtype,
+    uint16_t* __restrict__ out, int64_t n_rows, int64_t dim) {
+  const int64_t r = wave_row();
+  if (r >= n_rows) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const bool live = valid == nullptr || load_valid(valid, r, valid_dtype);
+  const uint16_t* b = bias + (live ? index[r] : 0) * dim;
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    u32x4 v[kBatch], w[kBatch];
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int c = c0 + k * kWave;
+      if (c < chunks) {
+        v[k] = ld16(rows + r * dim + c * 8);
+        if (live) w[k] = ld16(b + c * 8);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int c = c0 + k * kWave;
+      if (c < chunks) {
+        if (live) {
+          float f[8], g[8];
+          unpack8(v[k], f);
+          unpack8(w[k], g);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) f[i] += g[i];
+          v[k] = pack8(f);
+        }
+        st16(out + r * dim + c * 8, v[k]);
+      }
+    }
+  }
+}
+
+// Bias gradient: out[e,:] = sum of grad rows that belong to bank e, i.e. rows
+// row_index[seg_start[e] + i] (row_index == nullptr: seg_start[e] + i) for
+// i < seg_count[e].  A workgroup owns (bank, 512 columns, row split): its four
+// wavefronts take rows i = 4*(split + splits*j) + wave, their fp32 sums meet in
+// LDS in wavefront order, and with more than one split the per-split sums go to
+// `partial` [splits, E, dim] for segment_colsum_finish.  Fixed order throughout:
+// the result is reproducible bit for bit (no atomics).
+constexpr int kColsumCols = kWave * 8;
+__global__ __launch_bounds__(kRowBlock) void segment_colsum_kernel(
+    const uint16_t* __restrict__ grad, const int64_t* __restrict__ row_index,
+    const int64_t* __restrict__ seg_start, const int64_t* __restrict__ seg_count,
+    float* __restrict__ partial, uint16_t* __restrict__ out, int num_banks, int splits,
+    int64_t dim) {
+  __shared__ float red[kRowsPerBlock][kColsumCols];
+  const int e = blockIdx.x;
+  const int64_t col = static_cast<int64_t>(blockIdx.y) * kColsumCols + (threadIdx.x % kWave) * 8;
+  const int split = blockIdx.z;
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int64_t start = seg_start[e];
+  const int64_t count = seg_count[e];
+  const bool in_range = col < dim;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int64_t stride = static_cast<int64_t>(kRowsPerBlock) * splits;
+  for (int64_t i0 = static_cast<int64_t>(kRowsPerBlock) * split + wave; i0 < count;
+       i0 += stride * kBatch) {
+    u32x4 v[kBatch];
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int64_t i = i0 + k * stride;
+      if (i < count && in_range) {
+        const int64_t r = row_index == nullptr ? start + i : row_index[start + i];
+        v[k] = ld16(grad + r * dim + col);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      if (i0 + k * stride < count && in_range) {
+        float f[8];
+        unpack8(v[k], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] += f[j];
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) red[wave][lane * 8 + j] = acc[j];
+  __syncthreads();
+  if (wave == 0 && in_range) {
+    float sum[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      sum[j] = 0.0f;
+      for (int wv = 0; wv < kRowsPerBlock; ++wv) sum[j] += red[wv][lane * 8 + j];
+    }
+    if (splits == 1) {
+      st16(out + e * dim + col, pack8(sum));
+    } else {
+      float* dst = partial + (static_cast<int64_t>(split) * num_banks + e) * dim + col;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dst[j] = sum[j];
+    }
+  }
+}
+
+__global__ __launch_bounds__(kRowBlock) void segment_colsum_finish(
+    const float* __restrict__ partial, uint16_t* __restrict__ out, int64_t total, int splits) {
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * kRowBlock + threadIdx.x) * 8;
+  if (i >= total) return;
+  float sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int sp = 0; sp < splits; ++sp)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sum[j] += partial[sp * total + i + j];
+  st16(out + i, pack8(sum));
+}
+
 // Zero-fill of the padded rows that hold no assignment, for the source-major
 // kernels below: wavefront w looks at rows 64w .. 64w+63 (one per lane) and the
 // whole wavefront then clears each invalid one.
@@ -813,5 +929,40 @@ extern "C" int nestor_hip_path_scale_bwd(const void* grad_out, const void* in, c
     hipLaunchKernelGGL(path_scale_bwd_kernel<false>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),
                        0, s, grad_out, in, alpha, which, dest, grad_in, grad_alpha, num_tokens,
                        slots, num_out, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_bias_rows_fwd(const void* rows, const void* bias, const int64_t* index,
+                                        const void* valid, int32_t valid_dtype, void* out,
+                                        int64_t n_rows, int64_t dim, void* stream) {
+  if ((valid != nullptr && !dtype_ok(valid_dtype)) || dim <= 0 || dim % 8 != 0 || n_rows < 0)
+    return NESTOR_HIP_EINVAL;
+  if (n_rows == 0) return NESTOR_HIP_OK;
+  if (!rows || !bias || !index || !out) return NESTOR_HIP_EINVAL;
+  hipLaunchKernelGGL(bias_rows_fwd_kernel, dim3(row_blocks(n_rows)), dim3(kRowBlock), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(rows),
+                     static_cast<const uint16_t*>(bias), index, valid, valid_dtype,
+                     static_cast<uint16_t*>(out), n_rows, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_segment_colsum(const void* grad, const int64_t* row_index,
+                                         const int64_t* seg_start, const int64_t* seg_count,
+                                         float* partial, int32_t splits, void* out,
+                                         int32_t num_banks, int64_t dim, void* stream) {
+  if (dim <= 0 || dim % 8 != 0 || num_banks <= 0 || splits <= 0 || splits > 65535)
+    return NESTOR_HIP_EINVAL;
+  if (!grad || !seg_start || !seg_count || !out || (splits > 1 && !partial))
+    return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned col_blocks = static_cast<unsigned>(ceil_div(dim, kColsumCols));
+  hipLaunchKernelGGL(segment_colsum_kernel, dim3(num_banks, col_blocks, splits), dim3(kRowBlock),
+                     0, s, static_cast<const uint16_t*>(grad), row_index, seg_start, seg_count,
+                     partial, static_cast<uint16_t*>(out), num_banks, splits, dim);
+  if (splits > 1) {
+    const int64_t total = static_cast<int64_t>(num_banks) * dim;
+    hipLaunchKernelGGL(segment_colsum_finish, dim3(static_cast<unsigned>(ceil_div(total / 8, kRowBlock))),
+                       dim3(kRowBlock), 0, s, partial, static_cast<uint16_t*>(out), total, splits);
+  }
   return launch_status();
 }

@@ -98,11 +98,6 @@ def _bank_weights(
     return w_up, w_gate, w_down
 
 
-def _row_bias(bias_bank: Tensor, index: Tensor, valid: Tensor | None) -> Tensor:
-    rows = bias_bank.index_select(0, index)
-    return rows if valid is None else rows * valid.unsqueeze(1)
-
-
 def _expert_rows_padded(
     x: Tensor, experts: Sequence[nn.Module], plan: DispatchPlan, slots: int,
     dtype: torch.dtype, *, fused_gate: bool, stacked: "StackedExpertBank | None",
@@ -139,7 +134,10 @@ def _expert_rows_padded(
             stacked.b_up.to(dtype) if stacked is not None
             else torch.stack([e.layers[0].bias for e in experts]).to(dtype)
         )
-        hidden = hidden + _row_bias(b_up, plan.eid_pad, plan.pad_valid)
+        # one launch; the bias gradient is a segmented column sum over each bank's
+        # padded rows (the reference's one-hot GEMM, grouped_mm.py:159-177)
+        hidden = ops.bias_rows_op(hidden, b_up, plan.eid_pad, plan.pad_valid, None,
+                                  plan.padded_starts, plan.kept_counts)
     if gated:
         gate_rows = _plan_mm(x_pad, w_gate, plan)
         hidden = swiglu(hidden, gate_rows) if first.activation == "silu" else (
@@ -176,7 +174,9 @@ def grouped_expert_rows(
             stacked.b_down.to(dtype) if stacked is not None
             else torch.stack([e.layers[1].bias for e in experts]).to(dtype)
         )
-        routed = routed + _row_bias(b_down, flat_ids, None)
+        # routed rows are in token order: bank e owns rows order[raw_starts[e] + i]
+        routed = ops.bias_rows_op(routed, b_down, flat_ids, None, plan.order, plan.raw_starts,
+                                  plan.counts)
     return routed
 
 

@@ -757,6 +757,84 @@ def _(scores, choice_bias, mask, top_k, gate_mode):
 
 
 # --------------------------------------------------------------------------
+# Biased banks
+# --------------------------------------------------------------------------
+@torch.library.custom_op(f"{_NS}::bias_rows_fwd", mutates_args=(), device_types="cuda")
+def bias_rows_fwd(rows: Tensor, bias: Tensor, index: Tensor, valid: Tensor | None) -> Tensor:
+    rows = _bf16(rows, "rows")
+    bias = _bf16(bias, "bias")
+    out = torch.empty_like(rows)
+    v = None if valid is None else valid.contiguous()
+    _lib.call("nestor_hip_bias_rows_fwd", _ptr(rows), _ptr(bias), _ptr(index.contiguous()),
+              _ptr(v), 0 if v is None else _code(v.dtype), _ptr(out), rows.shape[0],
+              rows.shape[1], _stream(rows))
+    return out
+
+
+@bias_rows_fwd.register_fake
+def _(rows, bias, index, valid):
+    return torch.empty_like(rows)
+
+
+@torch.library.custom_op(f"{_NS}::segment_colsum", mutates_args=(), device_types="cuda")
+def segment_colsum(grad: Tensor, row_index: Tensor | None, seg_start: Tensor,
+                   seg_count: Tensor) -> Tensor:
+    """``out[e] = sum of grad rows of bank e`` (bf16 ``[E, dim]``), deterministic."""
+
+    grad = _bf16(grad, "grad")
+    num_banks = seg_start.shape[0]
+    dim = grad.shape[1]
+    rows = grad.shape[0] if row_index is None else row_index.shape[0]
+    # about 1024 rows per workgroup, so that few large banks still fill the device
+    splits = max(1, min(64, rows // (1024 * num_banks)))
+    partial = None
+    if splits > 1:
+        partial = torch.empty(splits, num_banks, dim, dtype=torch.float32, device=grad.device)
+    out = torch.empty(num_banks, dim, dtype=torch.bfloat16, device=grad.device)
+    ri = None if row_index is None else row_index.contiguous()
+    _lib.call("nestor_hip_segment_colsum", _ptr(grad), _ptr(ri), _ptr(seg_start.contiguous()),
+              _ptr(seg_count.contiguous()), _ptr(partial), splits, _ptr(out), num_banks, dim,
+              _stream(grad))
+    return out
+
+
+@segment_colsum.register_fake
+def _(grad, row_index, seg_start, seg_count):
+    return grad.new_empty(seg_start.shape[0], grad.shape[1])
+
+
+@torch.library.custom_op(f"{_NS}::bias_rows", mutates_args=(), device_types="cuda")
+def bias_rows_op(rows: Tensor, bias: Tensor, index: Tensor, valid: Tensor | None,
+                 row_index: Tensor | None, seg_start: Tensor, seg_count: Tensor) -> Tensor:
+    """``rows + bias[index]`` on the rows that hold an assignment.  ``row_index`` /
+    ``seg_start`` / ``seg_count`` describe each bank's rows for the bias gradient
+    (see :func:`segment_colsum`)."""
+
+    return bias_rows_fwd(rows, bias, index, valid)
+
+
+@bias_rows_op.register_fake
+def _(rows, bias, index, valid, row_index, seg_start, seg_count):
+    return torch.empty_like(rows)
+
+
+def _bias_rows_setup(ctx, inputs, output):
+    _rows, _bias, _index, _valid, row_index, seg_start, seg_count = inputs
+    ctx.save_for_backward(row_index, seg_start, seg_count)
+
+
+def _bias_rows_backward(ctx, grad):
+    row_index, seg_start, seg_count = ctx.saved_tensors
+    g_bias = None
+    if ctx.needs_input_grad[1]:
+        g_bias = segment_colsum(grad.contiguous(), row_index, seg_start, seg_count)
+    return grad, g_bias, None, None, None, None, None
+
+
+bias_rows_op.register_autograd(_bias_rows_backward, setup_context=_bias_rows_setup)
+
+
+# --------------------------------------------------------------------------
 # Path mix of the pool's summed layout
 # --------------------------------------------------------------------------
 def _mix_operands(alpha: Tensor, *tensors: Tensor) -> tuple[Tensor, ...]:

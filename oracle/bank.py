@@ -65,9 +65,28 @@ def swiglu_expert(x: Tensor, w_up: Tensor, w_gate: Tensor, w_down: Tensor) -> Te
     return (F.silu(x @ w_gate) * (x @ w_up)) @ w_down
 
 
+_ACTIVATIONS = {"silu": F.silu, "gelu": F.gelu, "relu": F.relu}
+
+
+def biased_expert(
+    x: Tensor, w_up: Tensor, w_gate: Tensor | None, w_down: Tensor, b_up: Tensor | None,
+    b_down: Tensor | None, activation: str = "silu",
+) -> Tensor:
+    """One expert of the native MoE banks: gated ``down(act(gate(x)) * up(x))`` with
+    biases on up and down only (nestor/scaling/blocks.py:251-312), or the pointwise
+    ``down(act(up(x)))`` when ``w_gate`` is None; stacked-layout weights."""
+
+    up = x @ w_up if b_up is None else x @ w_up + b_up
+    act = _ACTIVATIONS[activation]
+    hidden = act(x @ w_gate) * up if w_gate is not None else act(up)
+    out = hidden @ w_down
+    return out if b_down is None else out + b_down
+
+
 def gold_combine(
-    x: Tensor, w_up: Tensor, w_gate: Tensor, w_down: Tensor, expert_ids: Tensor,
-    weights: Tensor, group: int, row_kept: Tensor | None = None,
+    x: Tensor, w_up: Tensor, w_gate: Tensor | None, w_down: Tensor, expert_ids: Tensor,
+    weights: Tensor, group: int, row_kept: Tensor | None = None, *,
+    b_up: Tensor | None = None, b_down: Tensor | None = None, activation: str = "silu",
 ) -> Tensor:
     """Unrounded reference in the dtype of its inputs (use fp32 or fp64): every
     (token, slot) row through its expert, weighted, summed over each group of
@@ -82,7 +101,11 @@ def gold_combine(
         sel = torch.nonzero(flat_ids == e).squeeze(-1)
         if sel.numel() == 0:
             continue
-        y = swiglu_expert(x.index_select(0, tokens[sel]), w_up[e], w_gate[e], w_down[e])
+        y = biased_expert(
+            x.index_select(0, tokens[sel]), w_up[e], None if w_gate is None else w_gate[e],
+            w_down[e], None if b_up is None else b_up[e], None if b_down is None else b_down[e],
+            activation,
+        )
         rows = rows.index_add(0, sel, y)
     w = weights.reshape(-1, 1).to(x.dtype)
     if row_kept is not None:

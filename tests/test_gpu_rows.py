@@ -210,6 +210,45 @@ def test_path_scale_fwd_bwd(cuda, dtype, tokens, slots, cols, d):
         assert (t_alpha.grad[..., 1 - which] == 0).all()
 
 
+@pytest.mark.parametrize("tokens,slots,banks,dim", [(300, 2, 6, 40), (30000, 2, 4, 520), (4096, 1, 128, 1024)])
+def test_bias_rows_and_segment_colsum(cuda, tokens, slots, banks, dim):
+    """Bias add on padded rows (masked) and on routed rows, and the bias gradient as a
+    segmented column sum (one and several row splits) against an index_add."""
+
+    from nestor_amd import ops
+
+    ids, _ = routing(3, tokens, slots, banks)
+    want, got = _plan(ids, banks, cuda)
+    bias = torch.randn(banks, dim, generator=gen(1)).bfloat16()
+    # padded rows: slack rows keep their (zero) contents
+    rows = (torch.randn(want.rows_pad, dim, generator=gen(2)).bfloat16()
+            * want.pad_valid.unsqueeze(1))
+    ref = torch.where(want.pad_valid.bool().unsqueeze(1), rows + bias[want.eid_pad], rows)
+    tb = bias.to(cuda).requires_grad_(True)
+    out = ops.bias_rows_op(rows.to(cuda), tb, got.eid_pad, got.pad_valid, None,
+                           got.padded_starts, got.kept_counts)
+    assert torch.equal(out.cpu(), ref)
+    grad = torch.randn(want.rows_pad, dim, generator=gen(3)).bfloat16()
+    out.backward(grad.to(cuda))
+    valid = want.pad_valid.bool()
+    gref = torch.zeros(banks, dim).index_add_(0, want.eid_pad[valid], grad[valid].float())
+    torch.testing.assert_close(tb.grad.cpu().float(), gref, rtol=2 ** -7, atol=1e-3 * tokens ** 0.5)
+    # routed rows (token order): every row is live, bank e owns rows order[raw_starts[e] + i]
+    flat = ids.reshape(-1)
+    routed = torch.randn(tokens * slots, dim, generator=gen(4)).bfloat16()
+    tb2 = bias.to(cuda).requires_grad_(True)
+    out2 = ops.bias_rows_op(routed.to(cuda), tb2, flat.to(cuda), None, got.order, got.raw_starts,
+                            got.counts)
+    assert torch.equal(out2.cpu(), routed + bias[flat])
+    g2 = torch.randn(tokens * slots, dim, generator=gen(5)).bfloat16()
+    out2.backward(g2.to(cuda))
+    gref2 = torch.zeros(banks, dim).index_add_(0, flat, g2.float())
+    torch.testing.assert_close(tb2.grad.cpu().float(), gref2, rtol=2 ** -7, atol=1e-3 * tokens ** 0.5)
+    # bit-reproducible
+    again = ops.segment_colsum(g2.to(cuda), got.order, got.raw_starts, got.counts)
+    assert torch.equal(again, tb2.grad)
+
+
 def test_identity_round_trip(cuda):
     """combine(dispatch(x)) with unit weights sums each token's ``slots`` copies."""
 

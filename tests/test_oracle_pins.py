@@ -209,6 +209,36 @@ def test_path_scale_loop():
                                    rtol=2 ** -6, atol=5e-2)
 
 
+def test_biased_gold_per_token_modules():
+    """The biased / pointwise gold against per-token evaluation with ``F.linear`` on the
+    per-expert ``weight = owner[i].t()`` views, the way the reference's modules hold them
+    (nestor/scaling/blocks.py:306-312, expert_bank_stack.py:72-77)."""
+
+    import torch.nn.functional as F
+
+    tokens, slots, banks, d, h = 12, 2, 3, 6, 5
+    g = gen(5)
+    x = torch.randn(tokens, d, generator=g, dtype=torch.float64)
+    w_up, w_gate = (torch.randn(banks, d, h, generator=g, dtype=torch.float64) for _ in range(2))
+    w_down = torch.randn(banks, h, d, generator=g, dtype=torch.float64)
+    b_up = torch.randn(banks, h, generator=g, dtype=torch.float64)
+    b_down = torch.randn(banks, d, generator=g, dtype=torch.float64)
+    ids = torch.randint(0, banks, (tokens, slots), generator=g)
+    wts = torch.rand(tokens, slots, generator=g, dtype=torch.float64)
+    for gated, act in ((True, "silu"), (False, "gelu")):
+        out = obank.gold_combine(x, w_up, w_gate if gated else None, w_down, ids, wts, slots,
+                                 b_up=b_up, b_down=b_down, activation=act)
+        fn = getattr(F, act)
+        for t in range(tokens):
+            want = torch.zeros(d, dtype=torch.float64)
+            for s_ in range(slots):
+                e = int(ids[t, s_])
+                up = F.linear(x[t], w_up[e].t(), b_up[e])
+                hid = fn(F.linear(x[t], w_gate[e].t())) * up if gated else fn(up)
+                want += wts[t, s_] * F.linear(hid, w_down[e].t(), b_down[e])
+            torch.testing.assert_close(out[t, 0], want, rtol=1e-10, atol=1e-10)
+
+
 def test_segment_mm_and_bank_routes_agree():
     """grouped (padded) path == per-expert dense evaluation == sparse loop ==
     per-token loop, in fp32 where only summation order differs
