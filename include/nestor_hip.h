@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 5
+#define NESTOR_HIP_ABI_VERSION 6
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -258,6 +258,17 @@ int nestor_hip_router_topk(
     const uint8_t* mask /* nullable, [n] */,
     float* softmax_probs, int64_t* topk_indices, void* gates,
     int64_t n, int32_t num_choices, int32_t top_k, int32_t gate_mode,
+    void* stream);
+
+/* Gradient of the scores through gates (and through softmax_probs when grad_probs
+ * != NULL): what autograd derives from the reference's differentiable chain
+ * softmax -> gather -> scatter_add -> mask (nestor/backbones/nestor.py:565-590),
+ * fp32 with one rounding to the score dtype.  grad_gates [n, C] in the score
+ * dtype (nullable), grad_probs [n, C] fp32 (nullable), grad_scores [n, C]. */
+int nestor_hip_router_gates_bwd(
+    const void* scores, int32_t dtype, const int64_t* topk_indices,
+    const uint8_t* mask /* nullable */, const void* grad_gates, const float* grad_probs,
+    void* grad_scores, int64_t n, int32_t num_choices, int32_t top_k, int32_t gate_mode,
     void* stream);
 
 /* ------------------------------------------------------------------------

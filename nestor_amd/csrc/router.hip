@@ -86,6 +86,66 @@ __global__ __launch_bounds__(kRouterBlock) void router_topk_kernel(
   }
 }
 
+
+// Gradient of the scores through the gates (and, when grad_probs is given,
+// through softmax_probs), in the lane layout of the forward kernel:
+//   renorm: gate_j = softmax(scores[topk])_j  ->  dz_j = p_j * (dg_j - sum_i p_i dg_i)
+//   switch: gate_j = softmax(scores)[topk_j]  ->  ds_c = P_c * (dP_c - sum P dP), dP = dg on the top-k
+// with dg = grad_gates on the selected choices of rows the mask keeps, zero
+// elsewhere.  fp32 throughout, one rounding to the score dtype at the end -- the
+// eager chain (softmax backward in fp32, cast back) rounds at the same place.
+template <bool kF32>
+__global__ __launch_bounds__(kRouterBlock) void router_gates_bwd_kernel(
+    const void* __restrict__ scores, const int64_t* __restrict__ topk,
+    const uint8_t* __restrict__ mask, const void* __restrict__ grad_gates,
+    const float* __restrict__ grad_probs, void* __restrict__ grad_scores, int64_t n,
+    int num_choices, int top_k, int gate_mode, int group_shift) {
+  const int group = 1 << group_shift;
+  const int64_t gid = static_cast<int64_t>(blockIdx.x) * kRouterBlock + threadIdx.x;
+  const int64_t row = gid >> group_shift;
+  const int sub = static_cast<int>(gid & (group - 1));
+  const bool live = row < n && sub < num_choices;
+  const int dt = kF32 ? NESTOR_HIP_F32 : NESTOR_HIP_BF16;
+  const float ninf = -__builtin_inff();
+  float s = ninf, dg = 0.0f, dp = 0.0f;
+  bool taken = false;
+  if (live) {
+    s = load_scalar(scores, row * num_choices + sub, dt);
+    for (int j = 0; j < top_k; ++j) taken |= topk[row * top_k + j] == sub;
+    const bool valid = mask == nullptr || mask[row] != 0;
+    if (taken && valid && grad_gates != nullptr)
+      dg = load_scalar(grad_gates, row * num_choices + sub, dt);
+    if (grad_probs != nullptr) dp = grad_probs[row * num_choices + sub];
+  }
+  auto fmax_op = [](float a, float b) { return a > b ? a : b; };
+  auto fadd_op = [](float a, float b) { return a + b; };
+  const float m = group_reduce(s, group, fmax_op);
+  const float e = live ? expf(s - m) : 0.0f;
+  const float prob = e / group_reduce(e, group, fadd_op);
+  float ds = 0.0f;
+  if (gate_mode == 1) {
+    dp += dg;  // both paths go through the full softmax
+  } else {
+    const float m2 = group_reduce(taken ? s : ninf, group, fmax_op);
+    const float e2 = taken ? expf(s - m2) : 0.0f;
+    const float p2 = e2 / group_reduce(e2, group, fadd_op);
+    const float dot2 = group_reduce(p2 * dg, group, fadd_op);
+    ds = taken ? p2 * (dg - dot2) : 0.0f;
+  }
+  if (gate_mode == 1 || grad_probs != nullptr) {
+    const float dot = group_reduce(prob * dp, group, fadd_op);
+    ds += prob * (dp - dot);
+  }
+  if (live) {
+    if constexpr (kF32) {
+      reinterpret_cast<float*>(grad_scores)[row * num_choices + sub] = ds;
+    } else {
+      reinterpret_cast<uint16_t*>(grad_scores)[row * num_choices + sub] =
+          static_cast<uint16_t>(f32_to_bf16_bits(ds));
+    }
+  }
+}
+
 }  // namespace
 }  // namespace nestor
 
@@ -117,6 +177,32 @@ extern "C" int nestor_hip_router_topk(const void* scores, int32_t dtype,
     hipLaunchKernelGGL(router_topk_kernel<false>, dim3(blocks), dim3(kRouterBlock), 0, s,
                        scores, choice_bias, n_bias_rows, mask, softmax_probs, topk_indices,
                        gates, n, num_choices, top_k, gate_mode, shift);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_router_gates_bwd(const void* scores, int32_t dtype,
+                                           const int64_t* topk_indices, const uint8_t* mask,
+                                           const void* grad_gates, const float* grad_probs,
+                                           void* grad_scores, int64_t n, int32_t num_choices,
+                                           int32_t top_k, int32_t gate_mode, void* stream) {
+  if ((dtype != NESTOR_HIP_F32 && dtype != NESTOR_HIP_BF16) || num_choices <= 0 ||
+      num_choices > 64 || top_k <= 0 || top_k > num_choices || n < 0 ||
+      (gate_mode != 0 && gate_mode != 1))
+    return NESTOR_HIP_EINVAL;
+  if (n == 0) return NESTOR_HIP_OK;
+  if (!scores || !topk_indices || !grad_scores) return NESTOR_HIP_EINVAL;
+  int shift = 0;
+  while ((1 << shift) < num_choices) ++shift;
+  const unsigned blocks = static_cast<unsigned>(ceil_div(n << shift, kRouterBlock));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(router_gates_bwd_kernel<true>, dim3(blocks), dim3(kRouterBlock), 0, s,
+                       scores, topk_indices, mask, grad_gates, grad_probs, grad_scores, n,
+                       num_choices, top_k, gate_mode, shift);
+  else
+    hipLaunchKernelGGL(router_gates_bwd_kernel<false>, dim3(blocks), dim3(kRouterBlock), 0, s,
+                       scores, topk_indices, mask, grad_gates, grad_probs, grad_scores, n,
+                       num_choices, top_k, gate_mode, shift);
   return launch_status();
 }
 

@@ -756,6 +756,49 @@ def _(scores, choice_bias, mask, top_k, gate_mode):
             scores.new_empty(n, top_k, dtype=torch.long), torch.empty_like(scores)]
 
 
+@torch.library.custom_op(f"{_NS}::router_gates_bwd", mutates_args=(), device_types="cuda")
+def router_gates_bwd(
+    scores: Tensor, topk: Tensor, mask: Tensor | None, grad_gates: Tensor | None,
+    grad_probs: Tensor | None, gate_mode: int,
+) -> Tensor:
+    scores = scores.contiguous()
+    n, c = scores.shape
+    m = None if mask is None else mask.contiguous().view(torch.uint8)
+    gg = None if grad_gates is None else grad_gates.contiguous().to(scores.dtype)
+    gp = None if grad_probs is None else grad_probs.contiguous().float()
+    out = torch.empty_like(scores)
+    _lib.call(
+        "nestor_hip_router_gates_bwd", _ptr(scores), _code(scores.dtype), _ptr(topk.contiguous()),
+        _ptr(m), _ptr(gg), _ptr(gp), _ptr(out), n, c, topk.shape[1], gate_mode, _stream(scores),
+    )
+    return out
+
+
+@router_gates_bwd.register_fake
+def _(scores, topk, mask, grad_gates, grad_probs, gate_mode):
+    return torch.empty_like(scores)
+
+
+def _router_setup(ctx, inputs, output):
+    scores, _bias, mask, _top_k, gate_mode = inputs
+    _probs, topk, _gates = output
+    ctx.save_for_backward(scores, topk, mask)
+    ctx.gate_mode = gate_mode
+    ctx.set_materialize_grads(False)
+
+
+def _router_backward(ctx, grads):
+    grad_probs, _grad_topk, grad_gates = grads
+    scores, topk, mask = ctx.saved_tensors
+    if grad_probs is None and grad_gates is None:
+        return None, None, None, None, None
+    return (router_gates_bwd(scores, topk, mask, grad_gates, grad_probs, ctx.gate_mode),
+            None, None, None, None)
+
+
+router_topk.register_autograd(_router_backward, setup_context=_router_setup)
+
+
 # --------------------------------------------------------------------------
 # Biased banks
 # --------------------------------------------------------------------------

@@ -100,29 +100,20 @@ def route_scores(
 
     ``choice_bias`` is ``[C]`` or, for batched routers, ``[G, C]`` matching the
     second-to-last axis of ``scores``; ``mask`` has the shape of ``scores[..., 0]``.
-    The top-k and, when no gradient is needed, the gates come from the HIP
-    kernel; with gradients the gates are rebuilt from differentiable torch ops on
-    the kernel's indices, in the reference's op order.
+    One HIP launch; the op carries the gradient of the scores through the gates
+    and the softmax probabilities (one more launch), which is what autograd derives
+    from the reference's softmax / gather / scatter chain.
     """
 
     shape = scores.shape
     c = shape[-1]
-    flat = scores.reshape(-1, c)
     mode = 1 if gate_mode == "switch" else 0
     probs, topk, gates = ops.router_topk(
-        flat.detach(), choice_bias.detach().float().reshape(-1, c), mask.reshape(-1), top_k, mode
+        scores.reshape(-1, c), choice_bias.detach().float().reshape(-1, c), mask.reshape(-1),
+        top_k, mode,
     )
-    topk = topk.view(*shape[:-1], top_k)
-    if torch.is_grad_enabled() and scores.requires_grad:
-        softmax_probs = F.softmax(scores, dim=-1)
-        if gate_mode == "switch":
-            topk_gates = F.softmax(scores.float(), dim=-1).gather(-1, topk).to(scores.dtype)
-        else:
-            topk_gates = F.softmax(scores.gather(-1, topk).float(), dim=-1).to(scores.dtype)
-        dense = torch.zeros_like(scores).scatter_add(-1, topk, topk_gates)
-        dense = dense * mask.unsqueeze(-1).to(dense.dtype)
-        return softmax_probs, topk, dense
-    return probs.view(shape).to(_softmax_dtype(scores)), topk, gates.view(shape)
+    return (probs.view(shape).to(_softmax_dtype(scores)), topk.view(*shape[:-1], top_k),
+            gates.view(shape))
 
 
 class Router(nn.Module):

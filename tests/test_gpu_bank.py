@@ -25,7 +25,7 @@ def _hip_bank(cuda, x, w3, ids, weights, group, *, fused, capacity=0, autocast=F
 
     def call():
         return grouped_expert_combine(
-            tx, bank.expert_views(activation), ids.to(cuda), tw, group, fused_gate=True, stacked=bank,
+            tx, bank.expert_views(), ids.to(cuda), tw, group, fused_gate=True, stacked=bank,
             triton_index=True, triton_fused=fused, capacity=capacity,
         )
 

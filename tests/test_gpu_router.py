@@ -39,6 +39,53 @@ def test_router_topk_kernel(cuda, dtype, n, choices, k, mode):
         assert torch.equal(gates.cpu().float().sum(-1), mask.float())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("use_probs", [False, True])
+@pytest.mark.parametrize("n,choices,k,mode", [
+    (500, 8, 2, "renorm"), (500, 4, 1, "renorm"), (700, 16, 1, "switch"), (333, 15, 2, "switch"),
+    (257, 32, 2, "renorm"), (100, 64, 8, "switch"),
+])
+def test_router_score_gradient(cuda, dtype, use_probs, n, choices, k, mode):
+    """The op's score gradient (one launch) against autograd through the oracle's
+    softmax / gather / scatter chain in fp64 on the same selections."""
+
+    from nestor_amd import ops
+    from tests.helpers import rel_l2
+
+    g = gen(3 * n + choices)
+    scores = torch.randn(n, choices, generator=g).to(dtype)
+    bias = torch.randn(choices, generator=g) * 0.1
+    mask = torch.rand(n, generator=g) > 0.2
+    d_gates = torch.randn(n, choices, generator=g).to(dtype)
+    d_probs = torch.randn(n, choices, generator=g)
+    ts = scores.to(cuda).requires_grad_(True)
+    probs, topk, gates = ops.router_topk(ts, bias.to(cuda).view(1, -1), mask.to(cuda), k,
+                                         1 if mode == "switch" else 0)
+    loss = (gates.float() * d_gates.to(cuda).float()).sum()
+    if use_probs:
+        loss = loss + (probs * d_probs.to(cuda)).sum()
+    loss.backward()
+    # fp64 chain on the kernel's own selections (ties are the only way they could differ)
+    sd = scores.double().requires_grad_(True)
+    sel = topk.cpu()
+    if mode == "switch":
+        tg = torch.softmax(sd, -1).gather(-1, sel)
+    else:
+        tg = torch.softmax(sd.gather(-1, sel), -1)
+    dense = torch.zeros_like(sd).scatter_add(-1, sel, tg) * mask.unsqueeze(-1).double()
+    ref = (dense * d_gates.double()).sum()
+    if use_probs:
+        ref = ref + (torch.softmax(sd, -1) * d_probs.double()).sum()
+    ref.backward()
+    assert ts.grad.dtype == dtype
+    tol = 1e-5 if dtype == torch.float32 else 4e-3
+    assert rel_l2(ts.grad, sd.grad) < tol
+    if not use_probs:
+        assert (ts.grad.cpu()[~mask] == 0).all()
+        if k == 1 and mode == "renorm":
+            assert (ts.grad == 0).all()  # a renormalised top-1 gate is the constant 1
+
+
 def test_batched_private_routers_and_slots(cuda):
     """[T, G, Q] scores through one launch == G separate routers; slot ids are
     ``column * Q + expert`` and weights ``private_gate * column_gate``."""
