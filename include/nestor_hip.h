@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 6
+#define NESTOR_HIP_ABI_VERSION 7
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -269,6 +269,27 @@ int nestor_hip_router_gates_bwd(
     const void* scores, int32_t dtype, const int64_t* topk_indices,
     const uint8_t* mask /* nullable */, const void* grad_gates, const float* grad_probs,
     void* grad_scores, int64_t n, int32_t num_choices, int32_t top_k, int32_t gate_mode,
+    void* stream);
+
+/* Private slots of the pool (ExpertPoolMLP._private_slots,
+ * nestor/backbones/expert_pools.py:422-521): the k_a columns with the largest
+ * column gates per token (descending; equal gates lowest index first) -- or the
+ * caller's selected_in [T, k_a] -- and per selected column g its k_q chosen
+ * experts e = choices[t,g,i]: ids[t, j*k_q+i] = g*Q + e, weights = gates[t,g,e] *
+ * column_gates[t,g] rounded to `dtype`.  column_gates [T, G], gates [T, G, Q],
+ * choices [T, G, k_q]; G <= 64. */
+int nestor_hip_private_slots_fwd(
+    const void* column_gates, const void* gates, int32_t dtype, const int64_t* choices,
+    const int64_t* selected_in /* nullable */, int64_t* selected /* [T, k_a] */,
+    int64_t* ids /* [T, k_a*k_q] */, void* weights /* [T, k_a*k_q] */,
+    int64_t num_tokens, int32_t num_columns, int32_t num_experts, int32_t k_a, int32_t k_q,
+    void* stream);
+/* Gradients of the slot weights w.r.t. column_gates [T, G] and gates [T, G, Q]
+ * (dense, zero off the selected entries). */
+int nestor_hip_private_slots_bwd(
+    const void* grad_weights, const void* column_gates, const void* gates, int32_t dtype,
+    const int64_t* choices, const int64_t* selected, void* grad_column_gates, void* grad_gates,
+    int64_t num_tokens, int32_t num_columns, int32_t num_experts, int32_t k_a, int32_t k_q,
     void* stream);
 
 /* ------------------------------------------------------------------------

@@ -146,6 +146,101 @@ __global__ __launch_bounds__(kRouterBlock) void router_gates_bwd_kernel(
   }
 }
 
+// Private slots of the pool (ExpertPoolMLP._private_slots,
+// nestor/backbones/expert_pools.py:422-521): per token the k_a columns with the
+// largest column gates (descending, equal gates lowest index first; or the
+// caller's selection), and for each of them the column's k_q chosen experts:
+//   ids[t, j*k_q+i]     = g*Q + e            g = selected[t,j], e = choices[t,g,i]
+//   weights[t, j*k_q+i] = gates[t,g,e] * column_gates[t,g]   (rounded to the gate dtype)
+// One thread per token: the whole thing is a few dozen scalar loads.
+constexpr int kSlotsBlock = 128;
+
+template <bool kF32>
+__global__ __launch_bounds__(kSlotsBlock) void private_slots_fwd_kernel(
+    const void* __restrict__ column_gates, const void* __restrict__ gates,
+    const int64_t* __restrict__ choices, const int64_t* __restrict__ selected_in,
+    int64_t* __restrict__ selected, int64_t* __restrict__ ids, void* __restrict__ weights,
+    int64_t num_tokens, int num_columns, int num_experts, int k_a, int k_q) {
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kSlotsBlock + threadIdx.x;
+  if (t >= num_tokens) return;
+  const int dt = kF32 ? NESTOR_HIP_F32 : NESTOR_HIP_BF16;
+  uint64_t used = 0;
+  for (int j = 0; j < k_a; ++j) {
+    int g;
+    if (selected_in != nullptr) {
+      g = static_cast<int>(selected_in[t * k_a + j]);
+    } else {
+      float best = -__builtin_inff();
+      g = 0;
+      bool found = false;
+      for (int c = 0; c < num_columns; ++c) {
+        if ((used >> c) & 1) continue;
+        const float v = load_scalar(column_gates, t * num_columns + c, dt);
+        if (!found || v > best) {
+          best = v;
+          g = c;
+          found = true;
+        }
+      }
+      used |= 1ull << g;
+    }
+    selected[t * k_a + j] = g;
+    const float cg = load_scalar(column_gates, t * num_columns + g, dt);
+    for (int i = 0; i < k_q; ++i) {
+      const int64_t e = choices[(t * num_columns + g) * k_q + i];
+      const float pg = load_scalar(gates, (t * num_columns + g) * num_experts + e, dt);
+      const int64_t slot = (t * k_a + j) * k_q + i;
+      ids[slot] = static_cast<int64_t>(g) * num_experts + e;
+      const float w = pg * cg;
+      if constexpr (kF32) {
+        reinterpret_cast<float*>(weights)[slot] = w;
+      } else {
+        reinterpret_cast<uint16_t*>(weights)[slot] = static_cast<uint16_t>(f32_to_bf16_bits(w));
+      }
+    }
+  }
+}
+
+// Gradients of the slot weights: grad_column_gates[t,g] = sum_i round(dW * gate),
+// grad_gates[t,g,e] = round(dW * column_gate) on the selected entries, zero
+// elsewhere (the thread clears its token's rows first; a token's selected
+// columns are distinct, and so are a column's chosen experts).
+template <bool kF32>
+__global__ __launch_bounds__(kSlotsBlock) void private_slots_bwd_kernel(
+    const void* __restrict__ grad_weights, const void* __restrict__ column_gates,
+    const void* __restrict__ gates, const int64_t* __restrict__ choices,
+    const int64_t* __restrict__ selected, void* __restrict__ grad_column_gates,
+    void* __restrict__ grad_gates, int64_t num_tokens, int num_columns, int num_experts,
+    int k_a, int k_q) {
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kSlotsBlock + threadIdx.x;
+  if (t >= num_tokens) return;
+  const int dt = kF32 ? NESTOR_HIP_F32 : NESTOR_HIP_BF16;
+  auto store = [&](void* base, int64_t i, float v) {
+    if constexpr (kF32) {
+      reinterpret_cast<float*>(base)[i] = v;
+    } else {
+      reinterpret_cast<uint16_t*>(base)[i] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+    }
+  };
+  for (int c = 0; c < num_columns; ++c) store(grad_column_gates, t * num_columns + c, 0.0f);
+  for (int c = 0; c < num_columns * num_experts; ++c)
+    store(grad_gates, t * num_columns * num_experts + c, 0.0f);
+  for (int j = 0; j < k_a; ++j) {
+    const int64_t g = selected[t * k_a + j];
+    const float cg = load_scalar(column_gates, t * num_columns + g, dt);
+    float dcg = 0.0f;
+    for (int i = 0; i < k_q; ++i) {
+      const int64_t e = choices[(t * num_columns + g) * k_q + i];
+      const float pg = load_scalar(gates, (t * num_columns + g) * num_experts + e, dt);
+      const float dw = load_scalar(grad_weights, (t * k_a + j) * k_q + i, dt);
+      const float term = dw * pg;
+      dcg += kF32 ? term : round_bf16(term);
+      store(grad_gates, (t * num_columns + g) * num_experts + e, dw * cg);
+    }
+    store(grad_column_gates, t * num_columns + g, dcg);
+  }
+}
+
 }  // namespace
 }  // namespace nestor
 
@@ -203,6 +298,60 @@ extern "C" int nestor_hip_router_gates_bwd(const void* scores, int32_t dtype,
     hipLaunchKernelGGL(router_gates_bwd_kernel<false>, dim3(blocks), dim3(kRouterBlock), 0, s,
                        scores, topk_indices, mask, grad_gates, grad_probs, grad_scores, n,
                        num_choices, top_k, gate_mode, shift);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_private_slots_fwd(const void* column_gates, const void* gates,
+                                            int32_t dtype, const int64_t* choices,
+                                            const int64_t* selected_in, int64_t* selected,
+                                            int64_t* ids, void* weights, int64_t num_tokens,
+                                            int32_t num_columns, int32_t num_experts,
+                                            int32_t k_a, int32_t k_q, void* stream) {
+  if ((dtype != NESTOR_HIP_F32 && dtype != NESTOR_HIP_BF16) || num_columns <= 0 ||
+      num_columns > 64 || num_experts <= 0 || k_a <= 0 || k_a > num_columns || k_q <= 0 ||
+      k_q > num_experts || num_tokens < 0)
+    return NESTOR_HIP_EINVAL;
+  if (num_tokens == 0) return NESTOR_HIP_OK;
+  if (!column_gates || !gates || !choices || !selected || !ids || !weights)
+    return NESTOR_HIP_EINVAL;
+  const unsigned blocks = static_cast<unsigned>(ceil_div(num_tokens, kSlotsBlock));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(private_slots_fwd_kernel<true>, dim3(blocks), dim3(kSlotsBlock), 0, s,
+                       column_gates, gates, choices, selected_in, selected, ids, weights,
+                       num_tokens, num_columns, num_experts, k_a, k_q);
+  else
+    hipLaunchKernelGGL(private_slots_fwd_kernel<false>, dim3(blocks), dim3(kSlotsBlock), 0, s,
+                       column_gates, gates, choices, selected_in, selected, ids, weights,
+                       num_tokens, num_columns, num_experts, k_a, k_q);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_private_slots_bwd(const void* grad_weights, const void* column_gates,
+                                            const void* gates, int32_t dtype,
+                                            const int64_t* choices, const int64_t* selected,
+                                            void* grad_column_gates, void* grad_gates,
+                                            int64_t num_tokens, int32_t num_columns,
+                                            int32_t num_experts, int32_t k_a, int32_t k_q,
+                                            void* stream) {
+  if ((dtype != NESTOR_HIP_F32 && dtype != NESTOR_HIP_BF16) || num_columns <= 0 ||
+      num_columns > 64 || num_experts <= 0 || k_a <= 0 || k_a > num_columns || k_q <= 0 ||
+      k_q > num_experts || num_tokens < 0)
+    return NESTOR_HIP_EINVAL;
+  if (num_tokens == 0) return NESTOR_HIP_OK;
+  if (!grad_weights || !column_gates || !gates || !choices || !selected || !grad_column_gates ||
+      !grad_gates)
+    return NESTOR_HIP_EINVAL;
+  const unsigned blocks = static_cast<unsigned>(ceil_div(num_tokens, kSlotsBlock));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(private_slots_bwd_kernel<true>, dim3(blocks), dim3(kSlotsBlock), 0, s,
+                       grad_weights, column_gates, gates, choices, selected, grad_column_gates,
+                       grad_gates, num_tokens, num_columns, num_experts, k_a, k_q);
+  else
+    hipLaunchKernelGGL(private_slots_bwd_kernel<false>, dim3(blocks), dim3(kSlotsBlock), 0, s,
+                       grad_weights, column_gates, gates, choices, selected, grad_column_gates,
+                       grad_gates, num_tokens, num_columns, num_experts, k_a, k_q);
   return launch_status();
 }
 

@@ -799,6 +799,79 @@ def _router_backward(ctx, grads):
 router_topk.register_autograd(_router_backward, setup_context=_router_setup)
 
 
+@torch.library.custom_op(f"{_NS}::private_slots", mutates_args=(), device_types="cuda")
+def private_slots_op(
+    column_gates: Tensor, gates: Tensor, choices: Tensor, selected: Tensor | None, k_a: int,
+) -> list[Tensor]:
+    """``column_gates [T, G]``, ``gates [T, G, Q]``, ``choices [T, G, k_q]`` ->
+    ``[selected [T, k_a], ids [T, k_a*k_q], weights [T, k_a*k_q]]``; differentiable
+    in both gate tensors."""
+
+    cg = column_gates.contiguous()
+    pg = gates.contiguous()
+    if pg.dtype != cg.dtype:
+        raise TypeError("column gates and private gates must share one dtype")
+    ch = choices.contiguous()
+    tokens, columns, experts = pg.shape
+    k_q = ch.shape[2]
+    sel_in = None if selected is None else selected.contiguous()
+    sel = torch.empty(tokens, k_a, dtype=torch.long, device=cg.device)
+    ids = torch.empty(tokens, k_a * k_q, dtype=torch.long, device=cg.device)
+    weights = torch.empty(tokens, k_a * k_q, dtype=cg.dtype, device=cg.device)
+    _lib.call("nestor_hip_private_slots_fwd", _ptr(cg), _ptr(pg), _code(cg.dtype), _ptr(ch),
+              _ptr(sel_in), _ptr(sel), _ptr(ids), _ptr(weights), tokens, columns, experts, k_a,
+              k_q, _stream(cg))
+    return [sel, ids, weights]
+
+
+@private_slots_op.register_fake
+def _(column_gates, gates, choices, selected, k_a):
+    tokens, k_q = gates.shape[0], choices.shape[2]
+    return [gates.new_empty(tokens, k_a, dtype=torch.long),
+            gates.new_empty(tokens, k_a * k_q, dtype=torch.long),
+            gates.new_empty(tokens, k_a * k_q)]
+
+
+@torch.library.custom_op(f"{_NS}::private_slots_bwd", mutates_args=(), device_types="cuda")
+def private_slots_bwd(
+    grad_weights: Tensor, column_gates: Tensor, gates: Tensor, choices: Tensor, selected: Tensor,
+) -> list[Tensor]:
+    cg = column_gates.contiguous()
+    pg = gates.contiguous()
+    ch = choices.contiguous()
+    tokens, columns, experts = pg.shape
+    g_cg = torch.empty_like(cg)
+    g_pg = torch.empty_like(pg)
+    _lib.call("nestor_hip_private_slots_bwd", _ptr(grad_weights.contiguous().to(cg.dtype)),
+              _ptr(cg), _ptr(pg), _code(cg.dtype), _ptr(ch), _ptr(selected.contiguous()),
+              _ptr(g_cg), _ptr(g_pg), tokens, columns, experts, selected.shape[1], ch.shape[2],
+              _stream(cg))
+    return [g_cg, g_pg]
+
+
+@private_slots_bwd.register_fake
+def _(grad_weights, column_gates, gates, choices, selected):
+    return [torch.empty_like(column_gates), torch.empty_like(gates)]
+
+
+def _private_slots_setup(ctx, inputs, output):
+    column_gates, gates, choices, _selected, _k_a = inputs
+    ctx.save_for_backward(column_gates, gates, choices, output[0])
+    ctx.set_materialize_grads(False)
+
+
+def _private_slots_backward(ctx, grads):
+    grad_weights = grads[2]
+    if grad_weights is None:
+        return None, None, None, None, None
+    column_gates, gates, choices, selected = ctx.saved_tensors
+    g_cg, g_pg = private_slots_bwd(grad_weights, column_gates, gates, choices, selected)
+    return g_cg, g_pg, None, None, None
+
+
+private_slots_op.register_autograd(_private_slots_backward, setup_context=_private_slots_setup)
+
+
 # --------------------------------------------------------------------------
 # Biased banks
 # --------------------------------------------------------------------------

@@ -199,6 +199,13 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
             gates, choices = stacked
         gates = gates.reshape(num_tokens, self.num_groups, q)
         choices = choices.reshape(num_tokens, self.num_groups, k_q)
+        if (flat_group_gates.is_cuda and self.num_groups <= 64
+                and gates.dtype == flat_group_gates.dtype
+                and gates.dtype in (torch.bfloat16, torch.float32)):
+            # one launch (and one for both gate gradients) instead of top-k + gathers
+            picked = None if selected is None else selected.reshape(num_tokens, k_a)
+            selected, ids, weights = ops.private_slots_op(flat_group_gates, gates, choices, picked, k_a)
+            return ids, weights, selected
         if selected is None:
             selected = torch.topk(flat_group_gates, k_a, dim=-1).indices
         else:

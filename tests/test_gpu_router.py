@@ -116,6 +116,46 @@ def test_batched_private_routers_and_slots(cuda):
         assert torch.equal(one.gates, want.gates[0, :, gi])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("tokens,groups,q,k_a,k_q,given", [
+    (1000, 8, 4, 2, 1, False), (1000, 8, 4, 2, 1, True), (333, 32, 4, 2, 2, False),
+    (64, 3, 5, 3, 3, False), (500, 64, 2, 4, 1, False), (1, 1, 1, 1, 1, False),
+])
+def test_private_slots_op(cuda, dtype, tokens, groups, q, k_a, k_q, given):
+    """Slot ids / weights / selected columns in one launch: integer outputs and the
+    rounded weights equal the oracle's gather chain bit for bit; both gate gradients
+    equal autograd through that chain (single rounded products)."""
+
+    from nestor_amd import ops
+
+    g = gen(tokens + groups)
+    col_scores = torch.randn(tokens, groups, generator=g).to(dtype)  # bf16: equal gates occur
+    valid = torch.rand(tokens, generator=g) > 0.1
+    col = orouter.route(col_scores, torch.zeros(groups), k_a, "renorm", valid)
+    scores = torch.randn(tokens, groups, q, generator=g).to(dtype)
+    priv = orouter.route(scores, torch.zeros(groups, q), k_q, "switch",
+                         valid.unsqueeze(-1) & col.active_mask)
+    picked = col.topk_indices if given else None
+    cg = col.gates.detach().clone().requires_grad_(True)
+    pg = priv.gates.detach().clone().requires_grad_(True)
+    w_ids, w_weights, w_sel = orouter.private_slots(pg, priv.topk_indices, cg, k_a, picked)
+    d_w = torch.randn(tokens, k_a * k_q, generator=g).to(dtype)
+    w_weights.backward(d_w)
+    tcg = col.gates.to(cuda).requires_grad_(True)
+    tpg = priv.gates.to(cuda).requires_grad_(True)
+    sel, ids, weights = ops.private_slots_op(
+        tcg, tpg, priv.topk_indices.to(cuda), None if picked is None else picked.to(cuda), k_a)
+    assert torch.equal(sel.cpu(), w_sel)
+    assert torch.equal(ids.cpu(), w_ids)
+    assert torch.equal(weights.cpu(), w_weights.detach())
+    weights.backward(d_w.to(cuda))
+    if k_q == 1 or dtype == torch.float32:
+        torch.testing.assert_close(tcg.grad.cpu(), cg.grad, rtol=1e-6, atol=1e-7)
+    else:  # a k_q-term sum: fp32 here, bf16 partial sums in the eager chain
+        torch.testing.assert_close(tcg.grad.cpu().float(), cg.grad.float(), rtol=2 ** -6, atol=2e-2)
+    assert torch.equal(tpg.grad.cpu(), pg.grad)
+
+
 def test_pool_routing_matches_oracle_slots(cuda):
     """Pool routers + slot build on the GPU vs the oracle on the same scores."""
 
