@@ -247,6 +247,42 @@ def cpu_baseline(w, seed: int, target_seconds: float = 15.0) -> dict:
     }
 
 
+def fp8_probe(w, tensors, iters: int = 10) -> dict:
+    """The inference regime: the workload's two banks in e4m3 with per-channel scales,
+    forward only, at 64 / 256 / 1024 tokens (top-2 columns -> top-1 private, top-1
+    public).  Most experts see 0-8 rows, so a call is bound by streaming the weights of
+    the experts that got a row: bytes = 3*d*h per such expert (1 B per weight)."""
+
+    from nestor_amd import fp8
+
+    dev = tensors.x.device
+    d, h = w.d_model, w.hidden
+    banks = {"public": fp8.quantize_bank(*tensors.pub), "private": fp8.quantize_bank(*tensors.priv)}
+    g = torch.Generator(device=dev).manual_seed(5)
+    out = {}
+    for tokens in (64, 256, 1024):
+        x = tensors.x[:tokens]
+        cols = torch.rand(tokens, w.columns, generator=g, device=dev).topk(w.k_columns, -1).indices
+        priv_ids = cols * w.private + torch.randint(0, w.private, cols.shape, generator=g, device=dev)
+        pub_ids = torch.randint(0, w.public, (tokens, w.k_public), generator=g, device=dev)
+        calls = (("public", pub_ids, 1), ("private", priv_ids, priv_ids.shape[1]))
+        wts = {n: torch.rand(i.shape, generator=g, device=dev).to(torch.bfloat16) for n, i, _ in calls}
+
+        def run():
+            return [fp8.grouped_expert_combine_fp8(x, banks[n], i, wts[n], grp) for n, i, grp in calls]
+
+        ms = _event_ms(run, iters)
+        live = sum(int(torch.unique(i).numel()) for _, i, _ in calls)
+        nbytes = live * 3 * d * h
+        flops = 2.0 * 3 * d * h * sum(i.numel() for _, i, _ in calls)
+        out[str(tokens)] = {
+            "ms": round(ms, 4), "experts_with_rows": live, "weight_bytes": nbytes,
+            "gbs": round(nbytes / ms / 1e6, 1), "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+            "tokens_per_s": round(tokens / ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 2),
+        }
+    return out
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -259,6 +295,9 @@ def main() -> None:
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch one 2 GiB device copy and the dominant kernel twice, then exit: the "
                          "command to run under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
+    ap.add_argument("--fp8-probe", action="store_true",
+                    help="time the e4m3-weight forward at 64/256/1024 tokens and print one JSON "
+                         "line (HBM GB/s over the weights of the experts that received a row)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the expert MLP: run it with --gpus 1 "
@@ -276,6 +315,10 @@ def main() -> None:
     tensors = make_tensors(w, args.seed, dev)
     if args.traffic_probe:
         traffic_probe(w, tensors)
+        return
+    if args.fp8_probe:
+        print(json.dumps({"workload": f"{w.name}, e4m3 weights, forward only",
+                          "unit": "GB/s of weight bytes streamed", "tokens": fp8_probe(w, tensors)}))
         return
     column_router, pool = build_pool(w, tensors)
     params = list(column_router.parameters()) + list(pool.parameters())

@@ -133,6 +133,22 @@ __device__ __forceinline__ u32x4 fp8x8_to_bf16x8(u32x2 raw) {
   return pack8(f);
 }
 
+// The same widening through the packed convert instruction (an e4m3 value is
+// exactly representable in bf16, so no rounding happens).
+__device__ __forceinline__ u32x4 fp8x8_to_bf16x8_exact(u32x2 raw) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  u32x4 out;
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[w]), false);
+    const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(raw[w]), true);
+    out[2 * w] = __builtin_bit_cast(uint32_t, __builtin_convertvector(lo, bf16x2));
+    out[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(hi, bf16x2));
+  }
+  return out;
+}
+
 // Scheduling recipe for one fragment's worth of MFMAs: before MFMA m, let
 // through this MFMA's share of the LDS reads (0x100), LDS writes (0x200) and
 // global loads (0x010, any VMEM) that sit in the same scheduling region, so each memory
@@ -616,8 +632,8 @@ __device__ __forceinline__ void dma16(const void* src, uint32_t lds_addr) {
                : "s"(lds_addr), "v"(src)
                : "memory", "m0");
 }
-__device__ __forceinline__ uint32_t lds_byte_addr(const uint16_t* p) {
-  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((NESTOR_LDS const uint16_t*)p));
+__device__ __forceinline__ uint32_t lds_byte_addr(const void* p) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((NESTOR_LDS const void*)p));
 }
 // Eight consecutive contraction indices of one output index from a swizzled
 // contraction-major tile: two transposing reads kRowElems * 4 elements apart.
@@ -1019,6 +1035,173 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
 // Sixteen zero bytes: the DMA source of every piece that lies behind the end of
 // its segment.
 __device__ __align__(16) const uint16_t g_zero_piece[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+
+// ---------------------------------------------------------------------------
+// Weight-streaming kernel for e4m3 weights at a few rows per bank (the inference
+// regime: a bank call is bound by reading the weights of the banks that got a
+// row).  The register-staged kernel keeps one K step of 8 KiB of weights in
+// flight per workgroup, which is latency times occupancy = a quarter of the HBM
+// rate.  Here the e4m3 bytes go HBM -> LDS with the DMA path into a ring of
+// kStages K steps of 64 x 256 bytes, two workgroups per CU: ~96 KiB of weights
+// in flight per CU.  Weights are widened to bf16 in registers after a
+// transposing 8-bit LDS read (ds_read_b64_tr_b8: lanes 2r, 2r+1 of a 16-lane group
+// address 16 bytes of row r; lane j receives column j of the 8 x 16 byte block),
+// and the MFMA runs in bf16 as in the other kernels.
+//
+// A workgroup owns (tile, 256 output columns) and walks the tile's rows in
+// blocks of 32 * kMi rows, streaming the weight panel once per block: meant for
+// tiles that fit one block.
+// ---------------------------------------------------------------------------
+template <int kMi, int kStages>
+struct Fp8StreamCfg {
+  static constexpr int BN = 256, BK = 64;
+  static constexpr int ROWS = 32 * kMi;
+  static constexpr int A_BYTES = ROWS * BK * 2;   // bf16 activations, K-contiguous rows of 128 B
+  static constexpr int B_BYTES = BK * BN;         // e4m3 weights, rows of 256 B
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int A_LOADS = A_BYTES / 1024 / kWaves;  // DMA instructions per wavefront and K step
+  static constexpr int B_LOADS = B_BYTES / 1024 / kWaves;
+  static constexpr int LOADS = A_LOADS + B_LOADS;
+  static constexpr size_t LDS_BYTES = static_cast<size_t>(kStages) * STAGE_BYTES;
+  static_assert(A_BYTES % (1024 * kWaves) == 0, "whole DMA instructions per wavefront");
+};
+
+template <int kMi, int kStages>
+__global__ __launch_bounds__(kThreads, 2) void fp8w_stream_kernel(GemmParams p) {
+  using C = Fp8StreamCfg<kMi, kStages>;
+  extern __shared__ __align__(16) uint16_t lds[];
+  uint8_t* ring = reinterpret_cast<uint8_t*>(lds);
+  constexpr int BN = C::BN, BK = C::BK, S = kStages, NJ = 2, KK = BK / 16;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int tile = blockIdx.x / p.n_tiles;
+  const int nt = blockIdx.x % p.n_tiles;
+  const int32_t* tt = p.tile_table;
+  if (tile >= tt[3 * p.max_tiles]) return;
+  const int bank = tt[tile];
+  const int row0 = tt[p.max_tiles + tile];
+  const int nrows = tt[2 * p.max_tiles + tile];
+  const int64_t n0 = static_cast<int64_t>(nt) * BN;
+  if (bank < 0) {
+    const u32x4 zero = {0, 0, 0, 0};
+    for (int c = tid; c < nrows * (BN / 8); c += kThreads) {
+      const int row = c / (BN / 8);
+      st16(p.out + static_cast<int64_t>(row0 + row) * p.ldo + n0 + (c % (BN / 8)) * 8, zero);
+    }
+    return;
+  }
+  const int num_kt = static_cast<int>(p.K / BK);
+  const uint8_t* wq = static_cast<const uint8_t*>(p.b0) + static_cast<int64_t>(bank) * p.bank_stride;
+  const float* col_scale = p.scale + static_cast<int64_t>(bank) * p.N;
+
+  for (int rb = 0; rb < nrows; rb += C::ROWS) {
+    // ---- per-lane source addresses of this wavefront's DMA instructions ----
+    // A: instruction i moves rows 8*(wave + 4i) .. +7, lane -> (row, position);
+    // the position holds global piece (position ^ ((row >> 1) & 7)): conflict-free
+    // 128-bit fragment reads.  Rows past the tile re-read its last row.
+    const uint16_t* a_src[C::A_LOADS];
+#pragma unroll
+    for (int i = 0; i < C::A_LOADS; ++i) {
+      const int row = 8 * (wave + kWaves * i) + (lane >> 3);
+      const int piece = (lane & 7) ^ ((row >> 1) & 7);
+      const int r = rb + row < nrows ? rb + row : nrows - 1;
+      a_src[i] = p.a + static_cast<int64_t>(row0 + r) * p.lda + piece * 8;
+    }
+    // B: instruction i moves K rows 4*(wave + 4i) .. +3 of 256 bytes; position
+    // holds global piece (position ^ (2 * (k & 7))): conflict-free transposing reads.
+    const uint8_t* b_src[C::B_LOADS];
+#pragma unroll
+    for (int i = 0; i < C::B_LOADS; ++i) {
+      const int k = 4 * (wave + kWaves * i) + (lane >> 4);
+      const int piece = (lane & 15) ^ (2 * (k & 7));
+      b_src[i] = wq + static_cast<int64_t>(k) * p.ldb + n0 + piece * 16;
+    }
+    auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
+      kt = kt < num_kt ? kt : num_kt - 1;  // steps past the end re-fetch the last: uniform counts
+      uint8_t* sa = ring + stage * C::STAGE_BYTES;
+      uint8_t* sb = sa + C::A_BYTES;
+#pragma unroll
+      for (int i = 0; i < C::A_LOADS; ++i)
+        dma16(a_src[i] + static_cast<int64_t>(kt) * BK, lds_byte_addr(sa + (wave + kWaves * i) * 1024));
+#pragma unroll
+      for (int i = 0; i < C::B_LOADS; ++i)
+        dma16(b_src[i] + static_cast<int64_t>(kt) * BK * p.ldb,
+              lds_byte_addr(sb + (wave + kWaves * i) * 1024));
+    };
+
+    f32x16 acc[kMi][NJ];
+#pragma unroll
+    for (int i = 0; i < kMi; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+#pragma unroll
+    for (int t = 0; t + 1 < S; ++t) issue(t, t);
+
+    // fragment addressing
+    const int a_row = lane & 31, a_half = lane >> 5;
+    const int grp = lane >> 4, gi = lane & 15;
+    int cur = 0;
+    for (int kt = 0; kt < num_kt; ++kt) {
+      wait_vmcnt<(S - 2) * C::LOADS>();   // K step kt has landed (for this wavefront's transfers)
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();       // ... for everyone's, and step kt-1 is fully consumed
+      const int prev = cur == 0 ? S - 1 : cur - 1;
+      issue(kt + S - 1, prev);
+      const uint8_t* sa = ring + cur * C::STAGE_BYTES;
+      const uint8_t* sb = sa + C::A_BYTES;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        bf16x8 fa[kMi], fb[NJ];
+#pragma unroll
+        for (int i = 0; i < kMi; ++i) {
+          const int row = 32 * i + a_row;
+          const int piece = (2 * kk + a_half) ^ ((row >> 1) & 7);
+          fa[i] = *reinterpret_cast<const bf16x8*>(sa + row * 128 + piece * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          const int k = 16 * kk + 8 * (grp >> 1) + (gi >> 1);
+          const int piece = (4 * wave + 2 * j + (grp & 1)) ^ (2 * (k & 7));
+          typedef int v2i __attribute__((ext_vector_type(2)));
+          const v2i raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+              (NESTOR_LDS v2i*)(sb + k * BN + piece * 16 + 8 * (gi & 1)));
+          const u32x2 bits = {static_cast<uint32_t>(raw[0]), static_cast<uint32_t>(raw[1])};
+          fb[j] = __builtin_bit_cast(bf16x8, fp8x8_to_bf16x8_exact(bits));
+        }
+#pragma unroll
+        for (int i = 0; i < kMi; ++i)
+#pragma unroll
+          for (int j = 0; j < NJ; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+      }
+      cur = cur == S - 1 ? 0 : cur + 1;
+    }
+    wait_vmcnt<0>();                 // the re-fetched steps past the end
+    __builtin_amdgcn_s_barrier();    // before the next row block refills the ring
+
+    // ---- epilogue: scale per output column, round, store the tile's rows ----
+#pragma unroll
+    for (int i = 0; i < kMi; ++i) {
+      const int row = rb + 32 * i + (lane & 31);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t n = n0 + 64 * wave + 32 * j + 8 * q + 4 * (lane >> 5);
+          const f32x4 sc = *reinterpret_cast<const f32x4*>(col_scale + n);
+          const u32x2 packed = {pack_bf16x2(acc[i][j][4 * q] * sc[0], acc[i][j][4 * q + 1] * sc[1]),
+                                pack_bf16x2(acc[i][j][4 * q + 2] * sc[2], acc[i][j][4 * q + 3] * sc[3])};
+          if (row < nrows)
+            *reinterpret_cast<u32x2*>(p.out + static_cast<int64_t>(row0 + row) * p.ldo + n) = packed;
+        }
+    }
+  }
+}
 
 template <typename C>
 struct WgradLayout {
@@ -1434,6 +1617,24 @@ int launch_wgrad(const GemmParams& p, int32_t num_banks, void* stream) {
   return launch_status();
 }
 
+template <int kMi, int kStages>
+int launch_fp8_stream(GemmParams p, void* stream) {
+  using C = Fp8StreamCfg<kMi, kStages>;
+  p.n_tiles = static_cast<int>(p.N / C::BN);
+  const int64_t blocks = p.max_tiles * p.n_tiles;
+  if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fp8w_stream_kernel<kMi, kStages>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(C::LDS_BYTES));
+    configured = true;
+  }
+  hipLaunchKernelGGL((fp8w_stream_kernel<kMi, kStages>), dim3(static_cast<unsigned>(blocks)),
+                     dim3(kThreads), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
+  return launch_status();
+}
+
 }  // namespace
 }  // namespace nestor
 
@@ -1553,6 +1754,13 @@ extern "C" int nestor_hip_grouped_gemm_fp8w_nn(const void* a, const void* b_q,
   p.N = N;
   p.tile_table = tile_table;
   p.max_tiles = max_tiles;
+  // A few rows per bank: the call is bound by streaming the weights.  Average
+  // rows per bank from the static sizes (rows_pad holds 16 slack rows per bank).
+  const int64_t avg_rows = (rows_pad - 16 * static_cast<int64_t>(num_banks)) / num_banks;
+  int cfg = config_choice("NESTOR_HIP_FP8_CFG", avg_rows <= 24 ? 1 : avg_rows <= 56 ? 2 : 0);
+  if (K % 64 != 0 || N % 256 != 0) cfg = 0;
+  if (cfg == 1) return launch_fp8_stream<1, 4>(p, stream);
+  if (cfg == 2) return launch_fp8_stream<2, 3>(p, stream);
   return launch_rows<CfgSmall, kNNFp8W>(p, stream);
 }
 

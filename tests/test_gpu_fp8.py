@@ -66,3 +66,34 @@ def test_fp8_bank_at_1b_bank_shape(cuda):
                                         (bank.w_down, bank.s_down))]
     gold = obank.gold_combine(x.float(), *deq, ids, weights.float(), 1)
     assert rel_l2(out, gold) < 3e-2
+
+
+@pytest.mark.parametrize("cfg", ["0", "1", "2"])
+@pytest.mark.parametrize("tokens,slots,banks,K,N", [(300, 2, 6, 64, 256), (90, 1, 40, 512, 1024),
+                                                    (1000, 2, 5, 256, 512)])
+def test_fp8_weight_gemm_kernels_agree_with_dequantised_product(cuda, monkeypatch, cfg, tokens, slots,
+                                                                banks, K, N):
+    """The register-staged kernel (0) and the two weight-streaming configurations
+    (32 / 64 rows per pass over the weights), forced in turn: banks with zero rows,
+    with more rows than one pass covers, ragged last blocks.  Against the fp32 product
+    with the dequantised weights; slack rows stay exact zeros."""
+
+    from nestor_amd import ops
+    from nestor_amd.dispatch import dispatch_plan
+    from nestor_amd.fp8 import dequantize, quantize_per_channel
+    from oracle import bank as obank_
+    from oracle import plan as oplan
+    from tests.helpers import zipf_ids
+
+    monkeypatch.setenv("NESTOR_HIP_FP8_CFG", cfg)
+    ids = zipf_ids(2, tokens, slots, banks).reshape(-1)
+    want = oplan.dispatch_plan(ids, banks, slots, torch.bfloat16)
+    got = dispatch_plan(ids.to(cuda), banks, slots, torch.bfloat16)
+    a = (torch.randn(want.rows_pad, K, generator=gen(1)).bfloat16() * want.pad_valid.unsqueeze(1))
+    w = torch.randn(banks, K, N, generator=gen(2)) * 0.05
+    q, s = quantize_per_channel(w.to(cuda))
+    out = ops.grouped_gemm_fp8w_nn(a.to(cuda), q, s, got.tile_table)
+    ref = obank_.segment_mm(a.float(), dequantize(q, s).cpu(), want.offs)
+    assert out.dtype == torch.bfloat16 and out.shape == ref.shape
+    assert rel_l2(out, ref) < 4e-3  # bf16 output rounding only: the weights are the same e4m3 values
+    assert (out.cpu()[want.pad_valid == 0] == 0).all()
