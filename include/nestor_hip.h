@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 7
+#define NESTOR_HIP_ABI_VERSION 8
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -239,6 +239,17 @@ int nestor_hip_grouped_gemm_tn(
 int nestor_hip_grouped_gemm_fp8w_nn(
     const void* a, const void* b_q, const float* scale, void* out,
     int64_t rows_pad, int64_t K, int64_t N, int32_t num_banks,
+    const int32_t* tile_table, int64_t max_tiles, void* stream);
+/* The up and gate projections of an e4m3 bank and SwiGLU in one weight-streaming
+ * launch: hidden[r,n] = bf16( silu(gate) * up ), up = bf16(scale_up[bank,n] * a[r,:] @
+ * up_q[bank,:,n]), gate likewise, silu rounded to bf16 as in the unfused chain
+ * (nestor/backbones/triton_expert.py:172-175).  Meant for a few rows per bank
+ * (every 32 or 64 rows of a tile stream the weight panel once); K % 64 == 0 and
+ * H % 128 == 0, else NESTOR_HIP_EINVAL. */
+int nestor_hip_grouped_gemm_fp8w_upgate_swiglu(
+    const void* a, const void* up_q, const void* gate_q,
+    const float* scale_up, const float* scale_gate, void* hidden /* bf16 [rows_pad, H] */,
+    int64_t rows_pad, int64_t K, int64_t H, int32_t num_banks,
     const int32_t* tile_table, int64_t max_tiles, void* stream);
 
 /* ------------------------------------------------------------------------

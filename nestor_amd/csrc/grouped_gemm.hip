@@ -82,6 +82,7 @@ struct GemmParams {
   int64_t bank_stride;  // elements between banks of b0 / b1 (kTN: of out)
   int64_t ldb;
   const float* scale;   // [E, N] (kNNFp8W)
+  const float* scale2;  // [E, N] of the gate bank (fused e4m3 up|gate)
   uint16_t* out;
   int64_t ldo;
   uint16_t* out2;       // hidden (kNNUpGate)
@@ -1066,7 +1067,10 @@ struct Fp8StreamCfg {
   static_assert(A_BYTES % (1024 * kWaves) == 0, "whole DMA instructions per wavefront");
 };
 
-template <int kMi, int kStages>
+// kUpGate: the 256 weight columns of a K row are 128 of w_up and the same 128 of
+// w_gate; a wavefront accumulates 32 columns of each and the epilogue writes
+// hidden = silu(gate) * up with the bf16 rounding points of the unfused chain.
+template <int kMi, int kStages, bool kUpGate>
 __global__ __launch_bounds__(kThreads, 2) void fp8w_stream_kernel(GemmParams p) {
   using C = Fp8StreamCfg<kMi, kStages>;
   extern __shared__ __align__(16) uint16_t lds[];
@@ -1083,18 +1087,22 @@ __global__ __launch_bounds__(kThreads, 2) void fp8w_stream_kernel(GemmParams p) 
   const int bank = tt[tile];
   const int row0 = tt[p.max_tiles + tile];
   const int nrows = tt[2 * p.max_tiles + tile];
-  const int64_t n0 = static_cast<int64_t>(nt) * BN;
+  constexpr int kOutCols = kUpGate ? BN / 2 : BN;
+  const int64_t n0 = static_cast<int64_t>(nt) * kOutCols;
   if (bank < 0) {
     const u32x4 zero = {0, 0, 0, 0};
-    for (int c = tid; c < nrows * (BN / 8); c += kThreads) {
-      const int row = c / (BN / 8);
-      st16(p.out + static_cast<int64_t>(row0 + row) * p.ldo + n0 + (c % (BN / 8)) * 8, zero);
+    for (int c = tid; c < nrows * (kOutCols / 8); c += kThreads) {
+      const int row = c / (kOutCols / 8);
+      st16(p.out + static_cast<int64_t>(row0 + row) * p.ldo + n0 + (c % (kOutCols / 8)) * 8, zero);
     }
     return;
   }
   const int num_kt = static_cast<int>(p.K / BK);
   const uint8_t* wq = static_cast<const uint8_t*>(p.b0) + static_cast<int64_t>(bank) * p.bank_stride;
+  const uint8_t* wq2 =
+      kUpGate ? static_cast<const uint8_t*>(p.b1) + static_cast<int64_t>(bank) * p.bank_stride : wq;
   const float* col_scale = p.scale + static_cast<int64_t>(bank) * p.N;
+  const float* col_scale2 = kUpGate ? p.scale2 + static_cast<int64_t>(bank) * p.N : col_scale;
 
   for (int rb = 0; rb < nrows; rb += C::ROWS) {
     // ---- per-lane source addresses of this wavefront's DMA instructions ----
@@ -1116,7 +1124,10 @@ __global__ __launch_bounds__(kThreads, 2) void fp8w_stream_kernel(GemmParams p) 
     for (int i = 0; i < C::B_LOADS; ++i) {
       const int k = 4 * (wave + kWaves * i) + (lane >> 4);
       const int piece = (lane & 15) ^ (2 * (k & 7));
-      b_src[i] = wq + static_cast<int64_t>(k) * p.ldb + n0 + piece * 16;
+      if constexpr (kUpGate)
+        b_src[i] = (piece < 8 ? wq : wq2) + static_cast<int64_t>(k) * p.ldb + n0 + (piece & 7) * 16;
+      else
+        b_src[i] = wq + static_cast<int64_t>(k) * p.ldb + n0 + piece * 16;
     }
     auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
       kt = kt < num_kt ? kt : num_kt - 1;  // steps past the end re-fetch the last: uniform counts
@@ -1166,7 +1177,8 @@ __global__ __launch_bounds__(kThreads, 2) void fp8w_stream_kernel(GemmParams p) 
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
           const int k = 16 * kk + 8 * (grp >> 1) + (gi >> 1);
-          const int piece = (4 * wave + 2 * j + (grp & 1)) ^ (2 * (k & 7));
+          const int col_piece = kUpGate ? 8 * j + 2 * wave + (grp & 1) : 4 * wave + 2 * j + (grp & 1);
+          const int piece = col_piece ^ (2 * (k & 7));
           typedef int v2i __attribute__((ext_vector_type(2)));
           const v2i raw = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
               (NESTOR_LDS v2i*)(sb + k * BN + piece * 16 + 8 * (gi & 1)));
@@ -1188,17 +1200,36 @@ __global__ __launch_bounds__(kThreads, 2) void fp8w_stream_kernel(GemmParams p) 
 #pragma unroll
     for (int i = 0; i < kMi; ++i) {
       const int row = rb + 32 * i + (lane & 31);
-#pragma unroll
-      for (int j = 0; j < NJ; ++j)
+      uint16_t* dst = p.out + static_cast<int64_t>(row0 + row) * p.ldo;
+      if constexpr (kUpGate) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int64_t n = n0 + 64 * wave + 32 * j + 8 * q + 4 * (lane >> 5);
-          const f32x4 sc = *reinterpret_cast<const f32x4*>(col_scale + n);
-          const u32x2 packed = {pack_bf16x2(acc[i][j][4 * q] * sc[0], acc[i][j][4 * q + 1] * sc[1]),
-                                pack_bf16x2(acc[i][j][4 * q + 2] * sc[2], acc[i][j][4 * q + 3] * sc[3])};
-          if (row < nrows)
-            *reinterpret_cast<u32x2*>(p.out + static_cast<int64_t>(row0 + row) * p.ldo + n) = packed;
+          const int64_t n = n0 + 32 * wave + 8 * q + 4 * (lane >> 5);
+          const f32x4 su = *reinterpret_cast<const f32x4*>(col_scale + n);
+          const f32x4 sg = *reinterpret_cast<const f32x4*>(col_scale2 + n);
+          float h[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float u = round_bf16(acc[i][0][4 * q + e] * su[e]);
+            const float g = round_bf16(acc[i][1][4 * q + e] * sg[e]);
+            h[e] = round_bf16(g / (1.0f + __expf(-g))) * u;
+          }
+          const u32x2 packed = {pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3])};
+          if (row < nrows) *reinterpret_cast<u32x2*>(dst + n) = packed;
         }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int64_t n = n0 + 64 * wave + 32 * j + 8 * q + 4 * (lane >> 5);
+            const f32x4 sc = *reinterpret_cast<const f32x4*>(col_scale + n);
+            const u32x2 packed = {
+                pack_bf16x2(acc[i][j][4 * q] * sc[0], acc[i][j][4 * q + 1] * sc[1]),
+                pack_bf16x2(acc[i][j][4 * q + 2] * sc[2], acc[i][j][4 * q + 3] * sc[3])};
+            if (row < nrows) *reinterpret_cast<u32x2*>(dst + n) = packed;
+          }
+      }
     }
   }
 }
@@ -1617,20 +1648,20 @@ int launch_wgrad(const GemmParams& p, int32_t num_banks, void* stream) {
   return launch_status();
 }
 
-template <int kMi, int kStages>
+template <int kMi, int kStages, bool kUpGate>
 int launch_fp8_stream(GemmParams p, void* stream) {
   using C = Fp8StreamCfg<kMi, kStages>;
-  p.n_tiles = static_cast<int>(p.N / C::BN);
+  p.n_tiles = static_cast<int>(p.N / (kUpGate ? C::BN / 2 : C::BN));
   const int64_t blocks = p.max_tiles * p.n_tiles;
   if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fp8w_stream_kernel<kMi, kStages>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fp8w_stream_kernel<kMi, kStages, kUpGate>),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
                               static_cast<int>(C::LDS_BYTES));
     configured = true;
   }
-  hipLaunchKernelGGL((fp8w_stream_kernel<kMi, kStages>), dim3(static_cast<unsigned>(blocks)),
+  hipLaunchKernelGGL((fp8w_stream_kernel<kMi, kStages, kUpGate>), dim3(static_cast<unsigned>(blocks)),
                      dim3(kThreads), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
   return launch_status();
 }
@@ -1757,11 +1788,41 @@ extern "C" int nestor_hip_grouped_gemm_fp8w_nn(const void* a, const void* b_q,
   // A few rows per bank: the call is bound by streaming the weights.  Average
   // rows per bank from the static sizes (rows_pad holds 16 slack rows per bank).
   const int64_t avg_rows = (rows_pad - 16 * static_cast<int64_t>(num_banks)) / num_banks;
-  int cfg = config_choice("NESTOR_HIP_FP8_CFG", avg_rows <= 24 ? 1 : avg_rows <= 56 ? 2 : 0);
+  int cfg = config_choice("NESTOR_HIP_FP8_CFG", avg_rows <= 24 ? 1 : avg_rows <= 72 ? 2 : 0);
   if (K % 64 != 0 || N % 256 != 0) cfg = 0;
-  if (cfg == 1) return launch_fp8_stream<1, 4>(p, stream);
-  if (cfg == 2) return launch_fp8_stream<2, 3>(p, stream);
+  if (cfg == 1) return launch_fp8_stream<1, 4, false>(p, stream);
+  if (cfg == 2) return launch_fp8_stream<2, 3, false>(p, stream);
   return launch_rows<CfgSmall, kNNFp8W>(p, stream);
+}
+
+extern "C" int nestor_hip_grouped_gemm_fp8w_upgate_swiglu(
+    const void* a, const void* up_q, const void* gate_q, const float* scale_up,
+    const float* scale_gate, void* hidden, int64_t rows_pad, int64_t K, int64_t H,
+    int32_t num_banks, const int32_t* tile_table, int64_t max_tiles, void* stream) {
+  if (!dims_ok(rows_pad, K, H, num_banks, max_tiles) || K % 64 != 0 || H % 128 != 0)
+    return NESTOR_HIP_EINVAL;
+  if (rows_pad == 0) return NESTOR_HIP_OK;
+  if (!a || !up_q || !gate_q || !scale_up || !scale_gate || !hidden || !tile_table)
+    return NESTOR_HIP_EINVAL;
+  GemmParams p = {};
+  p.a = static_cast<const uint16_t*>(a);
+  p.lda = K;
+  p.b0 = up_q;
+  p.b1 = gate_q;
+  p.bank_stride = K * H;
+  p.ldb = H;
+  p.scale = scale_up;
+  p.scale2 = scale_gate;
+  p.out = static_cast<uint16_t*>(hidden);
+  p.ldo = H;
+  p.K = K;
+  p.N = H;
+  p.tile_table = tile_table;
+  p.max_tiles = max_tiles;
+  const int64_t avg_rows = (rows_pad - 16 * static_cast<int64_t>(num_banks)) / num_banks;
+  const int cfg = config_choice("NESTOR_HIP_FP8_CFG", avg_rows <= 24 ? 1 : 2);
+  if (cfg == 1) return launch_fp8_stream<1, 4, true>(p, stream);
+  return launch_fp8_stream<2, 3, true>(p, stream);
 }
 
 extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void* g,

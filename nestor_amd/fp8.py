@@ -64,9 +64,15 @@ def grouped_expert_combine_fp8(
         plan = dispatch_plan(expert_ids.reshape(-1), num_banks, slots, torch.bfloat16)
         x_pad = dispatch_rows(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots,
                               torch.bfloat16)
-        up = ops.grouped_gemm_fp8w_nn(x_pad, bank.w_up, bank.s_up, plan.tile_table)
-        gate = ops.grouped_gemm_fp8w_nn(x_pad, bank.w_gate, bank.s_gate, plan.tile_table)
-        hidden = swiglu(up, gate)
+        k, h = bank.w_up.shape[1], bank.w_up.shape[2]
+        if k % 64 == 0 and h % 128 == 0 and num_tokens * slots <= 72 * num_banks:
+            # a few rows per bank: both projections and SwiGLU in one pass over the weights
+            hidden = ops.grouped_gemm_fp8w_upgate_swiglu(
+                x_pad, bank.w_up, bank.w_gate, bank.s_up, bank.s_gate, plan.tile_table)
+        else:
+            up = ops.grouped_gemm_fp8w_nn(x_pad, bank.w_up, bank.s_up, plan.tile_table)
+            gate = ops.grouped_gemm_fp8w_nn(x_pad, bank.w_gate, bank.s_gate, plan.tile_table)
+            hidden = swiglu(up, gate)
         y_pad = ops.grouped_gemm_fp8w_nn(hidden, bank.w_down, bank.s_down, plan.tile_table)
         out = combine_rows(y_pad, plan.row_dest, plan.pad_src_row, plan.pad_valid,
                            weights.reshape(-1), group, x.dtype)

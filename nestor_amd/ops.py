@@ -645,6 +645,35 @@ def _(a, b_q, scale, tile_table):
     return a.new_empty(a.shape[0], b_q.shape[2])
 
 
+@torch.library.custom_op(f"{_NS}::grouped_gemm_fp8w_upgate_swiglu", mutates_args=(),
+                         device_types="cuda")
+def grouped_gemm_fp8w_upgate_swiglu(
+    a: Tensor, up_q: Tensor, gate_q: Tensor, scale_up: Tensor, scale_gate: Tensor,
+    tile_table: Tensor,
+) -> Tensor:
+    """``silu(gate) * up`` over e4m3 ``up_q`` / ``gate_q [E, K, H]`` in one weight-streaming
+    launch (``K % 64 == 0``, ``H % 128 == 0``)."""
+
+    a = _bf16(a, "a")
+    up_q, gate_q = up_q.contiguous(), gate_q.contiguous()
+    assert up_q.dtype == torch.float8_e4m3fn and gate_q.dtype == torch.float8_e4m3fn
+    rows_pad, k = a.shape
+    num_banks, kb, h = up_q.shape
+    assert kb == k and gate_q.shape == up_q.shape
+    out = torch.empty(rows_pad, h, dtype=torch.bfloat16, device=a.device)
+    _lib.call(
+        "nestor_hip_grouped_gemm_fp8w_upgate_swiglu", _ptr(a), _ptr(up_q), _ptr(gate_q),
+        _ptr(scale_up.contiguous()), _ptr(scale_gate.contiguous()), _ptr(out), rows_pad, k, h,
+        num_banks, _ptr(tile_table), _table_max_tiles(tile_table), _stream(a),
+    )
+    return out
+
+
+@grouped_gemm_fp8w_upgate_swiglu.register_fake
+def _(a, up_q, gate_q, scale_up, scale_gate, tile_table):
+    return a.new_empty(a.shape[0], up_q.shape[2])
+
+
 # Differentiable grouped matmul: out = a @ b[bank] per segment.
 @torch.library.custom_op(f"{_NS}::grouped_mm", mutates_args=(), device_types="cuda")
 def grouped_mm_op(

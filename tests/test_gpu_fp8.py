@@ -97,3 +97,35 @@ def test_fp8_weight_gemm_kernels_agree_with_dequantised_product(cuda, monkeypatc
     assert out.dtype == torch.bfloat16 and out.shape == ref.shape
     assert rel_l2(out, ref) < 4e-3  # bf16 output rounding only: the weights are the same e4m3 values
     assert (out.cpu()[want.pad_valid == 0] == 0).all()
+
+
+@pytest.mark.parametrize("cfg", ["1", "2"])
+@pytest.mark.parametrize("tokens,slots,banks,K,H", [(200, 2, 12, 128, 256), (64, 1, 30, 512, 1024),
+                                                    (700, 2, 5, 64, 128)])
+def test_fp8_fused_upgate_swiglu_equals_unfused(cuda, monkeypatch, cfg, tokens, slots, banks, K, H):
+    """One pass over both e4m3 projections with SwiGLU in the epilogue: the same
+    accumulation order and rounding points as two weight-streaming launches plus the
+    SwiGLU kernel, so the same bits; and within bf16 rounding of the fp32 chain."""
+
+    from nestor_amd import ops
+    from nestor_amd.dispatch import dispatch_plan
+    from nestor_amd.fp8 import dequantize, quantize_per_channel
+    from oracle import plan as oplan
+    from tests.helpers import zipf_ids
+
+    monkeypatch.setenv("NESTOR_HIP_FP8_CFG", cfg)
+    ids = zipf_ids(4, tokens, slots, banks).reshape(-1)
+    want = oplan.dispatch_plan(ids, banks, slots, torch.bfloat16)
+    got = dispatch_plan(ids.to(cuda), banks, slots, torch.bfloat16)
+    a = (torch.randn(want.rows_pad, K, generator=gen(1)).bfloat16() * want.pad_valid.unsqueeze(1)).to(cuda)
+    qu, su = quantize_per_channel((torch.randn(banks, K, H, generator=gen(2)) * 0.1).to(cuda))
+    qg, sg = quantize_per_channel((torch.randn(banks, K, H, generator=gen(3)) * 0.1).to(cuda))
+    fused = ops.grouped_gemm_fp8w_upgate_swiglu(a, qu, qg, su, sg, got.tile_table)
+    up = ops.grouped_gemm_fp8w_nn(a, qu, su, got.tile_table)
+    gate = ops.grouped_gemm_fp8w_nn(a, qg, sg, got.tile_table)
+    assert torch.equal(fused, ops.swiglu_split_fwd(up, gate))
+    upf = obank.segment_mm(a.cpu().float(), dequantize(qu, su).cpu(), want.offs)
+    gatef = obank.segment_mm(a.cpu().float(), dequantize(qg, sg).cpu(), want.offs)
+    ref = torch.nn.functional.silu(gatef) * upf
+    assert rel_l2(fused, ref) < 1e-2
+    assert (fused.cpu()[want.pad_valid == 0] == 0).all()
