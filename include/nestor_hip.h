@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 8
+#define NESTOR_HIP_ABI_VERSION 9
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -282,6 +282,14 @@ int nestor_hip_router_gates_bwd(
     void* grad_scores, int64_t n, int32_t num_choices, int32_t top_k, int32_t gate_mode,
     void* stream);
 
+/* Loss-free balancing statistic (Router.update_detached_parameters,
+ * nestor/backbones/nestor.py:613-615): counts[c] += number of (row, slot) pairs
+ * with mask[row] != 0 and topk_indices[row, slot] == c.  counts [C] int32 must be
+ * zeroed by the caller; integer sums, reproducible.  C <= 64. */
+int nestor_hip_router_choice_counts(
+    const int64_t* topk_indices /* [n, k] */, const uint8_t* mask /* nullable, [n] */,
+    int32_t* counts, int64_t n, int32_t top_k, int32_t num_choices, void* stream);
+
 /* Private slots of the pool (ExpertPoolMLP._private_slots,
  * nestor/backbones/expert_pools.py:422-521): the k_a columns with the largest
  * column gates per token (descending; equal gates lowest index first) -- or the
@@ -366,6 +374,28 @@ int nestor_hip_segment_colsum(
     const int64_t* seg_start, const int64_t* seg_count,
     float* partial /* nullable when splits == 1 */, int32_t splits,
     void* out /* bf16 [E, dim] */, int32_t num_banks, int64_t dim, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Packed column attention epilogue (gate_combine_slots,
+ * nestor/backbones/triton_packed.py:332-412,547-640): slot-layout rows from the
+ * packed output-GEMM rows.  out[s,:] = T(val) * T(gates[r]) with r = slot_rows[s],
+ * val = out_c[r,:] (+ bf16(bias[gid[r],:]), sum rounded to bf16), T = out_dtype.
+ * out_c bf16 [rows, dim], bias fp32 [G, dim] (nullable, then gid unused), gates
+ * fp32 [rows] (exactly 0 on alignment-tail rows).  Its row gather is
+ * nestor_hip_dispatch_rows_fwd (pack_rows, :650-676).
+ * ---------------------------------------------------------------------- */
+int nestor_hip_gate_slots_fwd(
+    const void* out_c, const float* bias, const int64_t* gid, const float* gates,
+    const int64_t* slot_rows, void* out, int32_t out_dtype, int64_t n_out, int64_t dim,
+    void* stream);
+/* grad_out_c[r,:] = bf16(gates[r] * g[slot_packed[r],:]); grad_gates[r] = sum_d g*val
+ * in fp32 when grad_gates != NULL.  The bias gradient is
+ * nestor_hip_segment_colsum over grad_out_c. */
+int nestor_hip_gate_slots_bwd(
+    const void* grad_slots, int32_t g_dtype, const void* out_c, const float* bias,
+    const int64_t* gid, const float* gates, const int64_t* slot_packed,
+    void* grad_out_c /* bf16 [rows, dim] */, float* grad_gates /* nullable */,
+    int64_t rows, int64_t dim, void* stream);
 
 #ifdef __cplusplus
 }

@@ -13,6 +13,8 @@ from nestor_amd.expert_kernels import (
     cat_cast,
     combine_rows,
     dispatch_rows,
+    gate_combine_slots,
+    pack_rows,
     swiglu,
     swiglu_fused,
 )
@@ -30,7 +32,8 @@ __all__ = [
     "DispatchPlan", "ExpertPoolMLP", "GROUPED_MM_ALIGN", "Router", "RouterOutput",
     "StackedBanksMixin", "StackedExpertBank", "SwigluExpert", "autocast_dtype",
     "bank_is_fusable", "build_dispatch_maps", "cat_cast", "combine_rows",
-    "consolidate_stacked_expert_banks", "dispatch_plan", "dispatch_rows",
-    "grouped_expert_combine", "grouped_expert_rows", "route_private_batched", "segment_mm",
+    "consolidate_stacked_expert_banks", "dispatch_plan", "dispatch_rows", "gate_combine_slots",
+    "grouped_expert_combine", "grouped_expert_rows", "pack_rows", "route_private_batched",
+    "segment_mm",
     "swiglu", "swiglu_fused",
 ]

@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_int32, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libnestor_hip.so"
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 F32 = 0
 BF16 = 1
@@ -67,6 +67,7 @@ _SIGNATURES: dict[str, list] = {
         _P, _I32, _P, _I32, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P,
     ],
     "nestor_hip_router_gates_bwd": [_P, _I32, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _P],
+    "nestor_hip_router_choice_counts": [_P, _P, _P, _I64, _I32, _I32, _P],
     "nestor_hip_private_slots_fwd": [
         _P, _P, _I32, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P,
     ],
@@ -77,6 +78,8 @@ _SIGNATURES: dict[str, list] = {
     "nestor_hip_path_mix_bwd": [_P, _P, _P, _P, _P, _P, _P, _I32, _I64, _I64, _P],
     "nestor_hip_bias_rows_fwd": [_P, _P, _P, _P, _I32, _P, _I64, _I64, _P],
     "nestor_hip_segment_colsum": [_P, _P, _P, _P, _P, _I32, _P, _I32, _I64, _P],
+    "nestor_hip_gate_slots_fwd": [_P, _P, _P, _P, _P, _P, _I32, _I64, _I64, _P],
+    "nestor_hip_gate_slots_bwd": [_P, _I32, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _P],
     "nestor_hip_path_scale_fwd": [_P, _P, _I32, _P, _P, _I32, _I64, _I32, _I32, _I64, _P],
     "nestor_hip_path_scale_bwd": [
         _P, _P, _P, _I32, _P, _P, _P, _I32, _I64, _I32, _I32, _I64, _P,

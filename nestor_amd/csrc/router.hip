@@ -241,6 +241,30 @@ __global__ __launch_bounds__(kSlotsBlock) void private_slots_bwd_kernel(
   }
 }
 
+// Loss-free balancing statistic (Router.update_detached_parameters,
+// nestor/backbones/nestor.py:613-615): counts[c] = number of (valid token, slot)
+// pairs whose choice is c.  Integer LDS histogram per workgroup, one integer
+// atomic per choice and workgroup into `counts` (which the caller zeroes):
+// integer sums, so the result does not depend on the order.
+__global__ __launch_bounds__(kRouterBlock) void choice_count_kernel(
+    const int64_t* __restrict__ topk, const uint8_t* __restrict__ mask,
+    int32_t* __restrict__ counts, int64_t n, int top_k, int num_choices) {
+  __shared__ int hist[64];
+  if (threadIdx.x < 64) hist[threadIdx.x] = 0;
+  __syncthreads();
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kRouterBlock;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kRouterBlock + threadIdx.x; i < n * top_k;
+       i += stride) {
+    const int64_t row = i / top_k;
+    if (mask != nullptr && mask[row] == 0) continue;
+    const int64_t c = topk[i];
+    if (c >= 0 && c < num_choices) atomicAdd(&hist[c], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x < num_choices && hist[threadIdx.x] != 0)
+    atomicAdd(&counts[threadIdx.x], hist[threadIdx.x]);
+}
+
 }  // namespace
 }  // namespace nestor
 
@@ -352,6 +376,20 @@ extern "C" int nestor_hip_private_slots_bwd(const void* grad_weights, const void
     hipLaunchKernelGGL(private_slots_bwd_kernel<false>, dim3(blocks), dim3(kSlotsBlock), 0, s,
                        grad_weights, column_gates, gates, choices, selected, grad_column_gates,
                        grad_gates, num_tokens, num_columns, num_experts, k_a, k_q);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_router_choice_counts(const int64_t* topk_indices, const uint8_t* mask,
+                                               int32_t* counts, int64_t n, int32_t top_k,
+                                               int32_t num_choices, void* stream) {
+  if (num_choices <= 0 || num_choices > 64 || top_k <= 0 || n < 0) return NESTOR_HIP_EINVAL;
+  if (n == 0) return NESTOR_HIP_OK;
+  if (!topk_indices || !counts) return NESTOR_HIP_EINVAL;
+  const int64_t want = ceil_div(n * top_k, kRouterBlock * 8);
+  const unsigned blocks = static_cast<unsigned>(want < 1 ? 1 : want > 1024 ? 1024 : want);
+  hipLaunchKernelGGL(choice_count_kernel, dim3(blocks), dim3(kRouterBlock), 0,
+                     static_cast<hipStream_t>(stream), topk_indices, mask, counts, n, top_k,
+                     num_choices);
   return launch_status();
 }
 

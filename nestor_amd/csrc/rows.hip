@@ -632,6 +632,115 @@ __global__ __launch_bounds__(kRowBlock) void segment_colsum_finish(
   st16(out + i, pack8(sum));
 }
 
+// Packed column attention epilogue (gate_combine_slots,
+// nestor/backbones/triton_packed.py:332-412): slot-layout rows from the packed
+// output-GEMM rows,
+//   out[s,:] = T(val) * T(gate[r]),  r = slot_rows[s],
+//   val = out_c[r,:] (+ bf16(bias[gid[r],:]), the sum rounded to bf16),
+// T the output dtype.  One wavefront per slot row.
+template <bool kOutF32>
+__global__ __launch_bounds__(kRowBlock) void gate_slots_fwd_kernel(
+    const uint16_t* __restrict__ out_c, const float* __restrict__ bias,
+    const int64_t* __restrict__ gid, const float* __restrict__ gates,
+    const int64_t* __restrict__ slot_rows, void* __restrict__ out, int64_t n_out, int64_t dim) {
+#pragma clang fp contract(off)
+  const int64_t s = wave_row();
+  if (s >= n_out) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const int64_t r = slot_rows[s];
+  const float gate = round_to<kOutF32>(gates[r]);
+  const float* b = bias != nullptr ? bias + gid[r] * dim : nullptr;
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    u32x4 v[kBatch];
+    f32x4 b0[kBatch], b1[kBatch];
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int c = c0 + k * kWave;
+      if (c < chunks) {
+        v[k] = ld16(out_c + r * dim + c * 8);
+        if (b != nullptr) {
+          b0[k] = *reinterpret_cast<const f32x4*>(b + c * 8);
+          b1[k] = *reinterpret_cast<const f32x4*>(b + c * 8 + 4);
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int c = c0 + k * kWave;
+      if (c < chunks) {
+        float f[8];
+        unpack8(v[k], f);
+        if (b != nullptr) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            f[i] = round_bf16(f[i] + round_bf16(b0[k][i]));
+            f[4 + i] = round_bf16(f[4 + i] + round_bf16(b1[k][i]));
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = f[i] * gate;
+        store8_from_f32<kOutF32>(out, s * dim + c * 8, f);
+      }
+    }
+  }
+}
+
+// grad_out_c[r,:] = bf16(gate[r] * g[slot_packed[r],:]);
+// grad_gates[r] = sum_d g * val (fp32) when asked for (:347-412).
+template <bool kGF32>
+__global__ __launch_bounds__(kRowBlock) void gate_slots_bwd_kernel(
+    const void* __restrict__ g, const uint16_t* __restrict__ out_c,
+    const float* __restrict__ bias, const int64_t* __restrict__ gid,
+    const float* __restrict__ gates, const int64_t* __restrict__ slot_packed,
+    uint16_t* __restrict__ g_out_c, float* __restrict__ g_gates, int64_t rows, int64_t dim) {
+#pragma clang fp contract(off)
+  const int64_t r = wave_row();
+  if (r >= rows) return;
+  const int lane = threadIdx.x % kWave;
+  const int chunks = static_cast<int>(dim / 8);
+  const int64_t sp = slot_packed[r];
+  const float gate = gates[r];
+  const float* b = bias != nullptr ? bias + gid[r] * dim : nullptr;
+  float dot = 0.0f;
+  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+    float go[kBatch][8];
+    u32x4 v[kBatch];
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int c = c0 + k * kWave;
+      if (c < chunks) {
+        load8_as_f32<kGF32>(g, sp * dim + c * 8, go[k]);
+        if (g_gates != nullptr) v[k] = ld16(out_c + r * dim + c * 8);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int c = c0 + k * kWave;
+      if (c < chunks) {
+        float o[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = gate * go[k][i];
+        st16(g_out_c + r * dim + c * 8, pack8(o));
+        if (g_gates != nullptr) {
+          float f[8];
+          unpack8(v[k], f);
+          if (b != nullptr) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] = round_bf16(f[i] + round_bf16(b[c * 8 + i]));
+          }
+#pragma unroll
+          for (int i = 0; i < 8; ++i) dot += go[k][i] * f[i];
+        }
+      }
+    }
+  }
+  if (g_gates != nullptr) {
+    dot = wave_sum(dot);
+    if (lane == 0) g_gates[r] = dot;
+  }
+}
+
 // Zero-fill of the padded rows that hold no assignment, for the source-major
 // kernels below: wavefront w looks at rows 64w .. 64w+63 (one per lane) and the
 // whole wavefront then clears each invalid one.
@@ -964,5 +1073,46 @@ extern "C" int nestor_hip_segment_colsum(const void* grad, const int64_t* row_in
     hipLaunchKernelGGL(segment_colsum_finish, dim3(static_cast<unsigned>(ceil_div(total / 8, kRowBlock))),
                        dim3(kRowBlock), 0, s, partial, static_cast<uint16_t*>(out), total, splits);
   }
+  return launch_status();
+}
+
+extern "C" int nestor_hip_gate_slots_fwd(const void* out_c, const float* bias, const int64_t* gid,
+                                         const float* gates, const int64_t* slot_rows, void* out,
+                                         int32_t out_dtype, int64_t n_out, int64_t dim,
+                                         void* stream) {
+  if (!dtype_ok(out_dtype) || dim <= 0 || dim % 8 != 0 || n_out < 0) return NESTOR_HIP_EINVAL;
+  if (n_out == 0) return NESTOR_HIP_OK;
+  if (!out_c || !gates || !slot_rows || !out || (bias != nullptr && !gid))
+    return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto* oc = static_cast<const uint16_t*>(out_c);
+  if (out_dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(gate_slots_fwd_kernel<true>, dim3(row_blocks(n_out)), dim3(kRowBlock), 0, s,
+                       oc, bias, gid, gates, slot_rows, out, n_out, dim);
+  else
+    hipLaunchKernelGGL(gate_slots_fwd_kernel<false>, dim3(row_blocks(n_out)), dim3(kRowBlock), 0, s,
+                       oc, bias, gid, gates, slot_rows, out, n_out, dim);
+  return launch_status();
+}
+
+extern "C" int nestor_hip_gate_slots_bwd(const void* grad_slots, int32_t g_dtype, const void* out_c,
+                                         const float* bias, const int64_t* gid, const float* gates,
+                                         const int64_t* slot_packed, void* grad_out_c,
+                                         float* grad_gates, int64_t rows, int64_t dim,
+                                         void* stream) {
+  if (!dtype_ok(g_dtype) || dim <= 0 || dim % 8 != 0 || rows < 0) return NESTOR_HIP_EINVAL;
+  if (rows == 0) return NESTOR_HIP_OK;
+  if (!grad_slots || !gates || !slot_packed || !grad_out_c || (grad_gates != nullptr && !out_c) ||
+      (bias != nullptr && !gid))
+    return NESTOR_HIP_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto* oc = static_cast<const uint16_t*>(out_c);
+  auto* goc = static_cast<uint16_t*>(grad_out_c);
+  if (g_dtype == NESTOR_HIP_F32)
+    hipLaunchKernelGGL(gate_slots_bwd_kernel<true>, dim3(row_blocks(rows)), dim3(kRowBlock), 0, s,
+                       grad_slots, oc, bias, gid, gates, slot_packed, goc, grad_gates, rows, dim);
+  else
+    hipLaunchKernelGGL(gate_slots_bwd_kernel<false>, dim3(row_blocks(rows)), dim3(kRowBlock), 0, s,
+                       grad_slots, oc, bias, gid, gates, slot_packed, goc, grad_gates, rows, dim);
   return launch_status();
 }

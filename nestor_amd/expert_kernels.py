@@ -29,6 +29,34 @@ def dispatch_rows(
     return ops.dispatch_rows_op(x, pad_token, pad_valid, row_dest, slots)
 
 
+def pack_rows(
+    x_flat: Tensor, tok_packed: Tensor, row_real: Tensor, slot_rows: Tensor, num_slots: int,
+    compute_dtype: torch.dtype,
+) -> Tensor:
+    """The packed column attention's row gather (nestor/backbones/triton_packed.py:650-676):
+    ``x_flat[tok_packed]`` cast to the compute dtype with alignment-tail rows
+    (``row_real`` False) zeroed; backward sums each token's ``num_slots`` rows through
+    ``slot_rows``.  The expert path's dispatch kernel under the attention path's names."""
+
+    _need_bf16(compute_dtype, "pack_rows")
+    return ops.dispatch_rows_op(x_flat, tok_packed, row_real.to(compute_dtype), slot_rows, num_slots)
+
+
+def gate_combine_slots(
+    out_c: Tensor, bo: Tensor | None, gid: Tensor | None, gates: Tensor, slot_rows: Tensor,
+    slot_packed: Tensor, out_dtype: torch.dtype,
+) -> Tensor:
+    """Output bias + upcast + gate + slot gather of the packed column attention
+    (nestor/backbones/triton_packed.py:720-747): ``[num_tokens * slots, dim]`` rows
+    ``(out_c[r] + bo[gid[r]]) * gates[r]`` with ``r = slot_rows[s]`` in ``out_dtype``."""
+
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise NotImplementedError(f"gate_combine_slots writes float32 or bfloat16, got {out_dtype}")
+    assert (bo is None) == (gid is None), "a bias needs the row -> group map"
+    return ops.gate_combine_slots_op(out_c, bo, gid, gates, slot_rows, slot_packed,
+                                     out_dtype == torch.float32)
+
+
 def cat_cast(a: Tensor, b: Tensor, dtype: torch.dtype) -> Tensor:
     """``torch.cat([a, b], -1).to(dtype)`` bit for bit; the backward writes each
     bank's fp32 gradient contiguously."""

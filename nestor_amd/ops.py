@@ -828,6 +828,25 @@ def _router_backward(ctx, grads):
 router_topk.register_autograd(_router_backward, setup_context=_router_setup)
 
 
+@torch.library.custom_op(f"{_NS}::router_choice_counts", mutates_args=(), device_types="cuda")
+def router_choice_counts(topk: Tensor, mask: Tensor | None, num_choices: int) -> Tensor:
+    """``[C]`` int32: how many (valid row, slot) pairs chose each entry."""
+
+    topk = topk.contiguous()
+    k = topk.shape[-1]
+    n = topk.numel() // k
+    m = None if mask is None else mask.contiguous().view(torch.uint8)
+    counts = torch.zeros(num_choices, dtype=torch.int32, device=topk.device)
+    _lib.call("nestor_hip_router_choice_counts", _ptr(topk), _ptr(m), _ptr(counts), n, k,
+              num_choices, _stream(topk))
+    return counts
+
+
+@router_choice_counts.register_fake
+def _(topk, mask, num_choices):
+    return topk.new_empty(num_choices, dtype=torch.int32)
+
+
 @torch.library.custom_op(f"{_NS}::private_slots", mutates_args=(), device_types="cuda")
 def private_slots_op(
     column_gates: Tensor, gates: Tensor, choices: Tensor, selected: Tensor | None, k_a: int,
@@ -1124,6 +1143,88 @@ def _path_scale_backward(ctx, grad_out):
 
 
 path_scale_op.register_autograd(_path_scale_backward, setup_context=_path_scale_setup)
+
+
+# --------------------------------------------------------------------------
+# Packed column attention epilogue
+# --------------------------------------------------------------------------
+@torch.library.custom_op(f"{_NS}::gate_slots_fwd", mutates_args=(), device_types="cuda")
+def gate_slots_fwd(out_c: Tensor, bias: Tensor | None, gid: Tensor | None, gates: Tensor,
+                   slot_rows: Tensor, out_f32: bool) -> Tensor:
+    out_c = _bf16(out_c, "out_c")
+    dim = out_c.shape[1]
+    n_out = slot_rows.shape[0]
+    out_dtype = torch.float32 if out_f32 else torch.bfloat16
+    out = torch.empty(n_out, dim, dtype=out_dtype, device=out_c.device)
+    b = None if bias is None else bias.contiguous().float()
+    gi = None if gid is None else gid.contiguous()
+    _lib.call("nestor_hip_gate_slots_fwd", _ptr(out_c), _ptr(b), _ptr(gi),
+              _ptr(gates.contiguous().float()), _ptr(slot_rows.contiguous()), _ptr(out),
+              _code(out_dtype), n_out, dim, _stream(out_c))
+    return out
+
+
+@gate_slots_fwd.register_fake
+def _(out_c, bias, gid, gates, slot_rows, out_f32):
+    return out_c.new_empty(slot_rows.shape[0], out_c.shape[1],
+                           dtype=torch.float32 if out_f32 else torch.bfloat16)
+
+
+@torch.library.custom_op(f"{_NS}::gate_slots_bwd", mutates_args=(), device_types="cuda")
+def gate_slots_bwd(grad_slots: Tensor, out_c: Tensor, bias: Tensor | None, gid: Tensor | None,
+                   gates: Tensor, slot_packed: Tensor, need_gates: bool) -> list[Tensor]:
+    grad_slots = grad_slots.contiguous()
+    out_c = _bf16(out_c, "out_c")
+    rows, dim = out_c.shape
+    g_out_c = torch.empty_like(out_c)
+    g_gates = torch.empty(rows if need_gates else 0, dtype=torch.float32, device=out_c.device)
+    b = None if bias is None else bias.contiguous().float()
+    gi = None if gid is None else gid.contiguous()
+    _lib.call("nestor_hip_gate_slots_bwd", _ptr(grad_slots), _code(grad_slots.dtype), _ptr(out_c),
+              _ptr(b), _ptr(gi), _ptr(gates.contiguous().float()), _ptr(slot_packed.contiguous()),
+              _ptr(g_out_c), _ptr(g_gates) if need_gates else None, rows, dim, _stream(out_c))
+    return [g_out_c, g_gates]
+
+
+@gate_slots_bwd.register_fake
+def _(grad_slots, out_c, bias, gid, gates, slot_packed, need_gates):
+    return [torch.empty_like(out_c),
+            out_c.new_empty(out_c.shape[0] if need_gates else 0, dtype=torch.float32)]
+
+
+@torch.library.custom_op(f"{_NS}::gate_combine_slots", mutates_args=(), device_types="cuda")
+def gate_combine_slots_op(out_c: Tensor, bias: Tensor | None, gid: Tensor | None, gates: Tensor,
+                          slot_rows: Tensor, slot_packed: Tensor, out_f32: bool) -> Tensor:
+    return gate_slots_fwd(out_c, bias, gid, gates, slot_rows, out_f32)
+
+
+@gate_combine_slots_op.register_fake
+def _(out_c, bias, gid, gates, slot_rows, slot_packed, out_f32):
+    return out_c.new_empty(slot_rows.shape[0], out_c.shape[1],
+                           dtype=torch.float32 if out_f32 else torch.bfloat16)
+
+
+def _gate_slots_setup(ctx, inputs, output):
+    out_c, bias, gid, gates, _slot_rows, slot_packed, _out_f32 = inputs
+    ctx.save_for_backward(out_c, bias, gid, gates, slot_packed)
+
+
+def _gate_slots_backward(ctx, grad_slots):
+    out_c, bias, gid, gates, slot_packed = ctx.saved_tensors
+    need_gates = ctx.needs_input_grad[3]
+    g_out_c, g_gates = gate_slots_bwd(grad_slots, out_c, bias, gid, gates, slot_packed, need_gates)
+    g_bias = None
+    if bias is not None and ctx.needs_input_grad[1]:
+        # rows of group e are those with gid == e: a stable sort groups them for the
+        # segmented column sum (the reference's deterministic mask-GEMM)
+        order = torch.argsort(gid, stable=True)
+        counts = torch.bincount(gid, minlength=bias.shape[0])
+        starts = torch.cumsum(counts, 0) - counts
+        g_bias = segment_colsum(g_out_c, order, starts, counts).to(bias.dtype)
+    return g_out_c, g_bias, None, (g_gates.to(gates.dtype) if need_gates else None), None, None, None
+
+
+gate_combine_slots_op.register_autograd(_gate_slots_backward, setup_context=_gate_slots_setup)
 
 
 # --------------------------------------------------------------------------

@@ -5,8 +5,10 @@ deterministic forward: score head, softmax, detached choice bias, top-k,
 ``renorm`` / ``switch`` gate, scatter, validity mask) and the batched evaluation
 of a layer's ``G`` private routers (nestor/backbones/batched_router.py:97-240).
 Everything after the score GEMM -- softmax, biased top-k, gates -- is one HIP
-launch for the whole ``[tokens, (G,) choices]`` block.  Exploration noise and
-the bias update belong to the training loop and are not part of this path.
+launch for the whole ``[tokens, (G,) choices]`` block, and the gradient of the
+scores is one more.  The loss-free balancing update of ``choice_bias``
+(nestor/backbones/nestor.py:596-634) takes its counts from a histogram launch.
+Exploration noise belongs to the training loop and is not part of this path.
 
 ``torch.topk`` leaves the order of equal scores open; this implementation (and
 its oracle) take equal biased scores lowest index first.
@@ -153,6 +155,23 @@ class Router(nn.Module):
             scores, self.choice_bias, self.num_choices_per_token, self.gate_mode, valid_token_mask
         )
         return RouterOutput(scores, probs, gates, topk, gates > 0, valid_token_mask)
+
+    @torch.no_grad()
+    def update_detached_parameters(self, topk_indices: Tensor, valid_token_mask: Tensor) -> None:
+        """Loss-free balancing (nestor/backbones/nestor.py:596-634): nudge the detached
+        ``choice_bias`` by ``bias_update_rate`` towards the mean load.  The per-choice
+        counts come from one histogram launch; the sum over data-parallel ranks the
+        reference offers under ``NESTOR_LOSSFREE_GLOBAL_COUNTS`` belongs to a
+        multi-GPU run and is not part of this build."""
+
+        if not self.loss_free_balancing:
+            return
+        counts = ops.router_choice_counts(
+            topk_indices.reshape(-1, topk_indices.shape[-1]), valid_token_mask.reshape(-1),
+            self.num_choices,
+        ).float()
+        error = counts.mean() - counts
+        self.choice_bias += self.bias_update_rate * torch.sign(error)
 
 
 def check_batchable(routers: list[Router]) -> None:

@@ -88,3 +88,15 @@ def private_slots(
         weights.reshape(num_tokens, k_a * k_q),
         selected,
     )
+
+
+def balancing_update(choice_bias: Tensor, topk: Tensor, valid: Tensor, rate: float) -> Tensor:
+    """Loss-free balancing step (nestor/backbones/nestor.py:613-634, single rank):
+    one-hot the selections, count valid tokens per choice, move every bias by
+    ``rate`` towards the mean load.  Returns the new bias."""
+
+    num_choices = choice_bias.shape[0]
+    one_hot = F.one_hot(topk, num_classes=num_choices).float()
+    assigned = one_hot.sum(dim=-2) * valid.unsqueeze(-1).float()
+    counts = assigned.reshape(-1, num_choices).sum(0)
+    return choice_bias + rate * torch.sign(counts.mean() - counts)

@@ -136,3 +136,15 @@ def path_scale_bwd(grad_out: Tensor, inp: Tensor, alpha: Tensor, which: int,
     leaves = [t.detach().clone().requires_grad_(True) for t in (inp, alpha)]
     path_scale(leaves[0], leaves[1], which, dest, num_out).backward(grad_out)
     return leaves[0].grad, leaves[1].grad
+
+
+def gate_combine_slots(out_c: Tensor, bo: Tensor | None, gid: Tensor | None, gates: Tensor,
+                       slot_rows: Tensor, out_dtype: torch.dtype) -> Tensor:
+    """Packed column attention epilogue, the eager chain its fused kernel is held to
+    (nestor/backbones/triton_packed.py:385-395): bias added in the GEMM dtype, the row
+    upcast to the stream dtype, multiplied by the row's gate in that dtype, gathered
+    into slot order."""
+
+    val = out_c if bo is None else out_c + bo.to(out_c.dtype).index_select(0, gid)
+    rows = val.to(out_dtype) * gates.to(out_dtype).unsqueeze(1)
+    return rows.index_select(0, slot_rows)

@@ -219,3 +219,24 @@ def test_score_linear_matches_linear(cuda, tokens, dim, heads, bias):
     # without a gradient on the rows the library path runs and gives the same values
     plain = score_linear(x.to(cuda), tw, tb)
     assert torch.equal(plain, out)
+
+
+@pytest.mark.parametrize("n,choices,k", [(5000, 16, 2), (100, 64, 8), (1, 3, 1), (70000, 32, 2)])
+def test_balancing_counts_and_bias_update(cuda, n, choices, k):
+    """Histogram of the selections of valid tokens (integer-exact) and the bias step."""
+
+    from nestor_amd import ops
+    from nestor_amd.router import Router
+
+    g = gen(n)
+    topk = torch.stack([torch.randperm(choices, generator=g)[:k] for _ in range(min(n, 512))])
+    topk = topk.repeat((n + 511) // 512, 1)[:n].view(1, n, k)
+    valid = (torch.rand(1, n, generator=g) > 0.25)
+    counts = ops.router_choice_counts(topk.to(cuda), valid.to(cuda), choices)
+    want = torch.bincount(topk[valid].reshape(-1), minlength=choices)
+    assert torch.equal(counts.cpu().long(), want)
+    router = Router(8, choices, k, [], loss_free_balancing=True, bias_update_rate=0.01).to(cuda)
+    router.choice_bias.copy_(torch.randn(choices, generator=g))
+    before = router.choice_bias.cpu().clone()
+    router.update_detached_parameters(topk.to(cuda), valid.to(cuda))
+    assert torch.equal(router.choice_bias.cpu(), orouter.balancing_update(before, topk, valid, 0.01))

@@ -249,6 +249,49 @@ def test_bias_rows_and_segment_colsum(cuda, tokens, slots, banks, dim):
     assert torch.equal(again, tb2.grad)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("biased", [False, True])
+@pytest.mark.parametrize("tokens,slots,groups,dim", [(300, 2, 8, 40), (1000, 2, 32, 512), (17, 4, 3, 1032)])
+def test_pack_rows_and_gate_combine_slots(cuda, out_dtype, biased, tokens, slots, groups, dim):
+    """The packed column attention's two row kernels under their reference names: the
+    gather equals the dispatch oracle bit for bit; the gated slot rows equal the eager
+    chain bit for bit; gradients of rows, gates and bias within rounding of autograd
+    through that chain."""
+
+    from nestor_amd import gate_combine_slots, pack_rows
+    from tests.helpers import rel_l2
+
+    ids, _ = routing(5, tokens, slots, groups)
+    want, got = _plan(ids, groups, cuda)
+    x = torch.randn(tokens, dim, generator=gen(1))
+    row_real = want.pad_valid.bool()
+    packed = pack_rows(x.to(cuda), got.pad_token, row_real.to(cuda), got.row_dest, slots, torch.bfloat16)
+    assert torch.equal(packed.cpu(), orows.dispatch_rows(x, want.pad_token, want.pad_valid, torch.bfloat16))
+    out_c = torch.randn(want.rows_pad, dim, generator=gen(2)).bfloat16()
+    gates = torch.rand(want.rows_pad, generator=gen(3)) * want.pad_valid.float()  # exactly 0 on tails
+    bo = torch.randn(groups, dim, generator=gen(4)) if biased else None
+    gid = want.eid_pad if biased else None
+    leaves = [t.clone().requires_grad_(True) for t in (out_c, gates)] + ([bo.clone().requires_grad_(True)] if biased else [])
+    ref = orows.gate_combine_slots(leaves[0], leaves[2] if biased else None, gid, leaves[1],
+                                   want.row_dest, out_dtype)
+    go = torch.randn(ref.shape, generator=gen(6)).to(out_dtype)
+    ref.backward(go)
+    t_out_c = out_c.to(cuda).requires_grad_(True)
+    t_gates = gates.to(cuda).requires_grad_(True)
+    t_bo = bo.to(cuda).requires_grad_(True) if biased else None
+    out = gate_combine_slots(t_out_c, t_bo, None if gid is None else gid.to(cuda), t_gates,
+                             got.row_dest, got.pad_src_row, out_dtype)
+    assert out.dtype == out_dtype and torch.equal(out.cpu(), ref.detach())
+    out.backward(go.to(cuda))
+    valid = want.pad_valid.bool()
+    torch.testing.assert_close(t_out_c.grad.cpu().float()[valid], leaves[0].grad.float()[valid],
+                               rtol=2 ** -6, atol=1e-3)
+    assert (t_out_c.grad.cpu()[~valid] == 0).all()  # zero gates zero the tail rows' gradient
+    assert rel_l2(t_gates.grad.cpu()[valid], leaves[1].grad[valid]) < 1e-2
+    if biased:
+        assert rel_l2(t_bo.grad, leaves[2].grad) < 1e-2
+
+
 def test_identity_round_trip(cuda):
     """combine(dispatch(x)) with unit weights sums each token's ``slots`` copies."""
 

@@ -49,6 +49,7 @@ def test_argument_checks_fail_before_any_launch():
     assert lib.nestor_hip_router_gates_bwd(null, 1, null, null, null, null, null, 4, 8, 9, 0, null) == -22  # k > C
     assert lib.nestor_hip_private_slots_fwd(null, null, 1, null, null, null, null, null, 4, 65, 4, 2, 1, null) == -22  # G > 64
     assert lib.nestor_hip_private_slots_bwd(null, null, null, 1, null, null, null, null, 4, 8, 4, 9, 1, null) == -22  # k_a > G
+    assert lib.nestor_hip_router_choice_counts(null, null, null, 4, 2, 65, null) == -22
     # pool epilogues and biased banks
     assert lib.nestor_hip_path_mix_fwd(null, null, null, null, 1, 4, 12, null) == -22  # dim % 8
     assert lib.nestor_hip_path_mix_bwd(null, null, null, null, null, null, null, 7, 4, 16, null) == -22  # dtype

@@ -239,6 +239,24 @@ def test_biased_gold_per_token_modules():
             torch.testing.assert_close(out[t, 0], want, rtol=1e-10, atol=1e-10)
 
 
+def test_gate_combine_slots_loop():
+    rows, dim, groups = 12, 8, 3
+    out_c = torch.randn(rows, dim, generator=gen(1)).bfloat16()
+    bo = torch.randn(groups, dim, generator=gen(2))
+    gid = torch.randint(0, groups, (rows,), generator=gen(3))
+    gates = torch.rand(rows, generator=gen(4))
+    slot_rows = torch.randperm(rows, generator=gen(5))[:9]
+    for dtype in (torch.float32, torch.bfloat16):
+        out = orows.gate_combine_slots(out_c, bo, gid, gates, slot_rows, dtype)
+        for s_, r in enumerate(slot_rows.tolist()):
+            for i in range(dim):
+                val = (out_c[r, i].float() + bo[gid[r], i].bfloat16().float()).bfloat16()
+                want = (val.to(dtype).float() * gates[r].to(dtype).float()).to(dtype)
+                assert out[s_, i] == want
+    plain = orows.gate_combine_slots(out_c, None, None, gates, slot_rows, torch.float32)
+    assert torch.equal(plain, out_c.float().index_select(0, slot_rows) * gates[slot_rows, None])
+
+
 def test_segment_mm_and_bank_routes_agree():
     """grouped (padded) path == per-expert dense evaluation == sparse loop ==
     per-token loop, in fp32 where only summation order differs
@@ -308,6 +326,22 @@ def test_router_library_routines_and_special_cases():
     tied = torch.tensor([[1.0, 3.0, 3.0, 0.0, 3.0]])
     assert orouter.stable_topk(tied, 2).tolist() == [[1, 2]]
     assert orouter.stable_topk(tied, 4).tolist() == [[1, 2, 4, 0]]
+
+
+def test_balancing_update_loop():
+    """Counting loop and the sign step: over-used choices go down by the rate, under-used up."""
+
+    topk = torch.tensor([[[0, 1], [0, 2], [0, 1], [3, 0]]])
+    valid = torch.tensor([[True, True, False, True]])
+    bias = torch.tensor([0.5, 0.0, -0.25, 1.0])
+    counts = [0, 0, 0, 0]
+    for t in range(4):
+        if valid[0, t]:
+            for c in topk[0, t].tolist():
+                counts[c] += 1
+    assert counts == [3, 1, 1, 1]  # mean 1.5
+    new = orouter.balancing_update(bias, topk, valid, 0.125)
+    assert new.tolist() == [0.375, 0.125, -0.125, 1.125]
 
 
 def test_private_slots_closed_form():
