@@ -37,6 +37,15 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 __device__ __forceinline__ float round_bf16(float f) {
   return bf16_bits_to_f32(f32_to_bf16_bits(f));
 }
+// silu(g) = g / (1 + exp(-g)) in fp32, rounded to bf16 (the activation's rounding
+// point in the reference chain).  The quotient goes through the hardware
+// reciprocal (1 ulp): the ten-instruction IEEE division sequence is a measurable
+// share of the fused up|gate epilogue, and the bf16 rounding that follows hides
+// the difference except on rounding ties.  Every kernel takes it from here, so the
+// fused and the unfused paths agree bit for bit.
+__device__ __forceinline__ float silu_rounded(float g) {
+  return round_bf16(g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)));
+}
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
 }

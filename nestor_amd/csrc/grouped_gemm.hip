@@ -559,7 +559,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
         unpack8(up, u);
         unpack8(gate, g);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) h[e] = round_bf16(g[e] / (1.0f + __expf(-g[e]))) * u[e];
+        for (int e = 0; e < 8; ++e) h[e] = silu_rounded(g[e]) * u[e];
         st16(p.out2 + r * p.ldo2 + n, pack8(h));
       }
     }
@@ -1003,7 +1003,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
         unpack8(up, u);
         unpack8(gate, g);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) h[e] = round_bf16(g[e] / (1.0f + __expf(-g[e]))) * u[e];
+        for (int e = 0; e < 8; ++e) h[e] = silu_rounded(g[e]) * u[e];
         st16(p.out2 + r * p.ldo2 + n, pack8(h));
       }
     }
@@ -1212,7 +1212,7 @@ __global__ __launch_bounds__(kThreads, 2) void fp8w_stream_kernel(GemmParams p) 
           for (int e = 0; e < 4; ++e) {
             const float u = round_bf16(acc[i][0][4 * q + e] * su[e]);
             const float g = round_bf16(acc[i][1][4 * q + e] * sg[e]);
-            h[e] = round_bf16(g / (1.0f + __expf(-g))) * u;
+            h[e] = silu_rounded(g) * u;
           }
           const u32x2 packed = {pack_bf16x2(h[0], h[1]), pack_bf16x2(h[2], h[3])};
           if (row < nrows) *reinterpret_cast<u32x2*>(dst + n) = packed;

@@ -115,11 +115,6 @@ __global__ __launch_bounds__(kRowBlock) void dispatch_bwd_kernel(
   }
 }
 
-__device__ __forceinline__ float silu_rounded(float g) {
-  // ATen silu: x / (1 + exp(-x)) in fp32, rounded to the bf16 input dtype.
-  return round_bf16(g / (1.0f + __expf(-g)));
-}
-
 __global__ __launch_bounds__(kRowBlock) void swiglu_fwd_kernel(
     const uint16_t* __restrict__ up, const uint16_t* __restrict__ gate,
     uint16_t* __restrict__ out, int64_t rows, int64_t hidden, int64_t stride_in,
@@ -154,9 +149,8 @@ __global__ __launch_bounds__(kRowBlock) void swiglu_bwd_kernel(
     unpack8(ld16(gate + r * stride_in + c * 8), g);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float e = __expf(-g[i]);
-      const float s = 1.0f / (1.0f + e);
-      const float act = round_bf16(g[i] / (1.0f + e));
+      const float s = __builtin_amdgcn_rcpf(1.0f + __expf(-g[i]));  // as silu_rounded forms it
+      const float act = round_bf16(g[i] * s);
       du[i] = go[i] * act;
       const float gact = round_bf16(go[i] * u[i]);
       // ATen silu_backward: dy * s * (1 + x * (1 - s)) in fp32.
