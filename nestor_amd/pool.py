@@ -53,6 +53,9 @@ def private_expert_hidden_dim(dim: int, num_groups_per_token: int, private_top_k
     return round_to_multiple_of_8(budget * dim / (num_groups_per_token * private_top_k))
 
 
+_KERNEL_STREAM_DTYPES = (torch.bfloat16, torch.float32)
+
+
 class ExpertPoolMLP(StackedBanksMixin, nn.Module):
     """Public + column-private SwiGLU expert pools behind layer-local routers."""
 
@@ -316,7 +319,10 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
         if public_update is None:
             return private_update.to(x.dtype), pub_out, priv_outs
         alpha = self._path_weights(x)
-        update = ops.path_mix_op(public_update, private_update, alpha)
+        if x.dtype in _KERNEL_STREAM_DTYPES:
+            update = ops.path_mix_op(public_update, private_update, alpha)
+        else:  # other stream dtypes: the reference's eager expression
+            update = (alpha[..., 0:1] * public_update + alpha[..., 1:2] * private_update).to(x.dtype)
         return update, pub_out, priv_outs
 
     def forward_per_slot(self, x: Tensor, valid_token_mask: Tensor, group_gates: Tensor,
@@ -345,6 +351,21 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
         per_slot = self._private_per_slot(flat_x, ids, weights)
         return self._gate_split(x, public_update, per_slot, pub_out, priv_outs, columns=selected)
 
+    def _gate_split_eager(self, x, public_update, per_slot, pub_out, priv_outs, columns):
+        """The reference's op chain (expert_pools.py:758-761,943-953), for stream dtypes
+        the kernels do not take."""
+
+        split = per_slot
+        if columns is not None:
+            index = columns.reshape(*x.shape[:-1], -1, 1).expand_as(per_slot)
+            split = per_slot.new_zeros(*x.shape[:-1], self.num_groups, self.dim).scatter_add(
+                -2, index, per_slot)
+        if public_update is None:
+            return None, split.to(x.dtype), pub_out, priv_outs
+        alpha = self._path_weights(x)
+        return ((alpha[..., 0:1] * public_update).to(x.dtype),
+                (alpha[..., 1:2].unsqueeze(-1) * split).to(x.dtype), pub_out, priv_outs)
+
     def _gate_split(self, x, public_update, per_slot, pub_out, priv_outs, columns=None):
         """Outputs of the split layouts from the per-slot rows ``[n or B,S, k_a, d]``.
         ``columns [n, k_a]`` scatters the slots onto the ``G`` column streams
@@ -353,6 +374,8 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
 
         lead = x.shape[:-1]
         per_slot = per_slot.reshape(*lead, -1, self.dim)
+        if x.dtype not in _KERNEL_STREAM_DTYPES:
+            return self._gate_split_eager(x, public_update, per_slot, pub_out, priv_outs, columns)
         width = per_slot.shape[-2] if columns is None else self.num_groups
         dest = None if columns is None else columns.reshape(*lead, -1)
         if public_update is None:
