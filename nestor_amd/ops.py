@@ -949,8 +949,11 @@ def segment_colsum(grad: Tensor, row_index: Tensor | None, seg_start: Tensor,
     num_banks = seg_start.shape[0]
     dim = grad.shape[1]
     rows = grad.shape[0] if row_index is None else row_index.shape[0]
-    # about 1024 rows per workgroup, so that few large banks still fill the device
-    splits = max(1, min(64, rows // (1024 * num_banks)))
+    # enough workgroups to fill the device (a few thousand), each with at least
+    # ~128 rows to sum
+    col_blocks = -(-dim // 512)
+    want = -(-4096 // (num_banks * col_blocks))
+    splits = max(1, min(64, want, rows // (128 * num_banks)))
     partial = None
     if splits > 1:
         partial = torch.empty(splits, num_banks, dim, dtype=torch.float32, device=grad.device)
