@@ -406,9 +406,10 @@ extern "C" int nestor_hip_index_build(
                            static_cast<int64_t>(NESTOR_HIP_ROW_ALIGN) * num_banks;
   if (rows_pad != want_pad || rows_pad > INT32_MAX) return NESTOR_HIP_EINVAL;
   if (max_tiles < nestor_hip_max_tiles(rows_pad, num_banks)) return NESTOR_HIP_EINVAL;
-  if (!order || !counts || !raw_starts || !padded_starts || !offs || !row_dest ||
-      !pad_token || !pad_src_row || !eid_pad || !pad_valid || !tile_table || !workspace ||
-      (rows > 0 && !expert_ids))
+  // the per-row arrays of an empty batch are empty: their pointers may be null
+  if (!counts || !raw_starts || !padded_starts || !offs || !pad_token || !pad_src_row ||
+      !eid_pad || !pad_valid || !tile_table || !workspace ||
+      (rows > 0 && (!expert_ids || !order || !row_dest)))
     return NESTOR_HIP_EINVAL;
   if (workspace_bytes < nestor_hip_index_build_workspace_bytes(rows, num_banks))
     return NESTOR_HIP_ENOSPC;

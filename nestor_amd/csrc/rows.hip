@@ -996,11 +996,10 @@ extern "C" int nestor_hip_path_scale_fwd(const void* in, const void* alpha, int3
                                          int64_t num_tokens, int32_t slots, int32_t num_out,
                                          int64_t dim, void* stream) {
   if (!dtype_ok(dtype) || dim <= 0 || dim % 8 != 0 || num_tokens < 0 || slots <= 0 ||
-      slots > 64 || num_out <= 0 || (which != 0 && which != 1) ||
-      (dest == nullptr && num_out != slots))
+      slots > 64 || num_out <= 0 || (which != 0 && which != 1))
     return NESTOR_HIP_EINVAL;
-  if (num_tokens == 0) return NESTOR_HIP_OK;
-  if (!in || !alpha || !out) return NESTOR_HIP_EINVAL;
+  if (num_tokens == 0) return NESTOR_HIP_OK;  // empty tensors may come with null pointers
+  if (!in || !alpha || !out || (dest == nullptr && num_out != slots)) return NESTOR_HIP_EINVAL;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t rows = num_tokens * ((num_out + 7) / 8);  // wavefronts: 8 streams each
   if (dtype == NESTOR_HIP_F32)
@@ -1018,11 +1017,12 @@ extern "C" int nestor_hip_path_scale_bwd(const void* grad_out, const void* in, c
                                          int32_t slots, int32_t num_out, int64_t dim,
                                          void* stream) {
   if (!dtype_ok(dtype) || dim <= 0 || dim % 8 != 0 || num_tokens < 0 || slots <= 0 ||
-      slots > 64 || num_out <= 0 || (which != 0 && which != 1) ||
-      (dest == nullptr && num_out != slots))
+      slots > 64 || num_out <= 0 || (which != 0 && which != 1))
     return NESTOR_HIP_EINVAL;
   if (num_tokens == 0) return NESTOR_HIP_OK;
-  if (!grad_out || !in || !alpha || !grad_in || !grad_alpha) return NESTOR_HIP_EINVAL;
+  if (!grad_out || !in || !alpha || !grad_in || !grad_alpha ||
+      (dest == nullptr && num_out != slots))
+    return NESTOR_HIP_EINVAL;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == NESTOR_HIP_F32)
     hipLaunchKernelGGL(path_scale_bwd_kernel<true>, dim3(row_blocks(num_tokens)), dim3(kRowBlock),

@@ -98,6 +98,24 @@ def _bank_weights(
     return w_up, w_gate, w_down
 
 
+def _empty_result(x: Tensor, experts: Sequence[nn.Module], stacked, dtype: torch.dtype,
+                  out_rows: tuple[int, ...], out_dtype: torch.dtype, *extra: Tensor) -> Tensor:
+    """Result of a bank call over zero tokens: no rows, but still a function of the
+    inputs and the bank, so that a backward pass gives every parameter its (zero)
+    gradient as the reference's empty tensors do."""
+
+    first = experts[0]
+    gated = bool(getattr(first, "gated", False))
+    w_up, w_gate, w_down = _bank_weights(experts, stacked, dtype, gated)
+    tie = w_up.sum() + w_down.sum() + x.sum().to(dtype)
+    if w_gate is not None:
+        tie = tie + w_gate.sum()
+    for t in extra:
+        tie = tie + t.sum().to(dtype)
+    out = x.new_zeros(*out_rows, w_down.shape[-1], dtype=out_dtype)
+    return out + (tie * 0).to(out_dtype)
+
+
 def _expert_rows_padded(
     x: Tensor, experts: Sequence[nn.Module], plan: DispatchPlan, slots: int,
     dtype: torch.dtype, *, fused_gate: bool, stacked: "StackedExpertBank | None",
@@ -163,6 +181,8 @@ def grouped_expert_rows(
     del triton_index
     num_tokens, slots = expert_ids.shape
     dtype = _gemm_dtype(x)
+    if num_tokens == 0:
+        return _empty_result(x, experts, stacked, dtype, (0,), dtype)
     flat_ids = expert_ids.reshape(-1)
     plan = dispatch_plan(flat_ids, len(experts), slots, dtype)
     out_pad = _expert_rows_padded(
@@ -214,6 +234,9 @@ def grouped_expert_combine(
     del triton_index
     num_tokens, slots = expert_ids.shape
     assert slots % group == 0, "group must divide the slot count"
+    if num_tokens == 0:
+        return _empty_result(x, experts, stacked, _gemm_dtype(x), (0, slots // group), x.dtype,
+                             weights)
     fusable = bank_is_fusable(list(experts), fused_gate)
     if not fusable:
         if capacity > 0:

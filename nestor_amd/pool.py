@@ -280,7 +280,7 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
     def _public_update(self, flat_x: Tensor, public_output: RouterOutput, num_tokens: int) -> Tensor:
         ids, weights = self._public_slots(public_output, num_tokens)
         return self._bank(flat_x, self._public_bank(), self.stacked_public, ids, weights,
-                          self.public_top_k).reshape(num_tokens, -1)
+                          self.public_top_k).reshape(num_tokens, self.dim)
 
     def _private_per_slot(self, flat_x: Tensor, ids: Tensor, weights: Tensor) -> Tensor:
         return self._bank(flat_x, self._private_bank(), self.stacked_private, ids, weights,
@@ -333,10 +333,10 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
             x, valid_token_mask, group_gates, group_active_mask
         )
         ids, weights, _ = self._private_slots(
-            priv_outs, flat_gates, n, selected=slot_groups.reshape(n, -1), stacked=stacked
+            priv_outs, flat_gates, n, selected=slot_groups.reshape(n, self.num_groups_per_token), stacked=stacked
         )
         per_slot = self._private_per_slot(flat_x, ids, weights).view(
-            x.shape[0], x.shape[1], -1, self.dim
+            x.shape[0], x.shape[1], self.num_groups_per_token, self.dim
         )
         return self._gate_split(x, public_update, per_slot, pub_out, priv_outs)
 
@@ -373,11 +373,11 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
         weights scale both parts.  One launch per part."""
 
         lead = x.shape[:-1]
-        per_slot = per_slot.reshape(*lead, -1, self.dim)
+        per_slot = per_slot.reshape(*lead, self.num_groups_per_token, self.dim)
         if x.dtype not in _KERNEL_STREAM_DTYPES:
             return self._gate_split_eager(x, public_update, per_slot, pub_out, priv_outs, columns)
         width = per_slot.shape[-2] if columns is None else self.num_groups
-        dest = None if columns is None else columns.reshape(*lead, -1)
+        dest = None if columns is None else columns.reshape(*lead, self.num_groups_per_token)
         if public_update is None:
             if dest is None:
                 return None, per_slot.to(x.dtype), pub_out, priv_outs

@@ -278,3 +278,34 @@ def test_biased_bank_vs_gold(cuda, gated, activation, tokens, d, h, banks, slots
         assert rel_l2(getattr(bank, n).grad, leaf.grad) < TOL, n
     if gated:
         assert rel_l2(bank.w_gate.grad, w_gate.grad) < TOL
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("tokens", [0, 1, 3])
+def test_empty_and_tiny_batches(cuda, tokens, fused):
+    """No tokens: an empty result and zero gradients for every bank tensor (a sequence
+    slice can be empty); one and three tokens: most banks hold no row."""
+
+    from nestor_amd import StackedExpertBank, grouped_expert_combine
+
+    banks, d, h, slots = 4, 64, 128, 2
+    w3 = bank_weights(1, banks, d, h, 0.05, torch.bfloat16)
+    bank = StackedExpertBank.from_tensors(*[t.clone() for t in w3]).to(cuda)
+    ids = torch.randint(0, banks, (tokens, slots), generator=gen(tokens))
+    weights = torch.rand(tokens, slots, generator=gen(1)).bfloat16()
+    x = torch.randn(tokens, d, generator=gen(2)).bfloat16()
+    tx = x.to(cuda).requires_grad_(True)
+    tw = weights.to(cuda).requires_grad_(True)
+    out = grouped_expert_combine(tx, bank.expert_views(), ids.to(cuda), tw, slots, fused_gate=True,
+                                 stacked=bank, triton_index=True, triton_fused=fused)
+    assert out.shape == (tokens, 1, d) and out.dtype == torch.bfloat16
+    out.float().sum().backward()
+    assert tx.grad.shape == x.shape and tw.grad.shape == weights.shape
+    for t in (bank.w_up, bank.w_gate, bank.w_down):
+        assert t.grad is not None and torch.isfinite(t.grad.float()).all()
+    if tokens == 0:
+        assert all(float(t.grad.float().abs().sum()) == 0.0 for t in (bank.w_up, bank.w_gate, bank.w_down))
+    else:
+        ref, gx, gw, gw3 = _gold(x, w3, ids, weights, slots, torch.ones(tokens, 1, d))
+        assert rel_l2(out, ref) < TOL and rel_l2(tx.grad, gx) < TOL and rel_l2(tw.grad, gw) < TOL
+        assert rel_l2(bank.w_down.grad, gw3[2]) < TOL

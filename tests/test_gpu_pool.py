@@ -109,3 +109,24 @@ def test_pool_grads_reach_every_parameter(cuda):
     for n, p in pool.named_parameters():
         assert p.grad is not None and torch.isfinite(p.grad).all(), n
     assert x.grad is not None and torch.isfinite(x.grad).all()
+
+
+def test_pool_on_an_empty_sequence_slice(cuda):
+    """Zero tokens (the reference calls the pool on sequence slices): empty outputs of
+    the right shapes from all three layouts, and a backward pass that reaches the banks."""
+
+    pool = _pool(cuda, True).train()
+    x = torch.zeros(2, 0, 40, device=cuda, dtype=torch.bfloat16, requires_grad=True)
+    valid = torch.ones(2, 0, dtype=torch.bool, device=cuda)
+    gates = torch.zeros(2, 0, 4, device=cuda, dtype=torch.bfloat16)
+    active = torch.zeros(2, 0, 4, dtype=torch.bool, device=cuda)
+    slot_groups = torch.zeros(2, 0, 2, dtype=torch.long, device=cuda)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        update, _, _ = pool(x, valid, gates, active)
+        pub_s, priv_s, _, _ = pool.forward_per_slot(x, valid, gates, active, slot_groups)
+        pub_g, priv_g, _, _ = pool.forward_per_group(x, valid, gates, active)
+    assert update.shape == (2, 0, 40) and pub_s.shape == (2, 0, 40) and pub_g.shape == (2, 0, 40)
+    assert priv_s.shape == (2, 0, 2, 40) and priv_g.shape == (2, 0, 4, 40)
+    (update.sum() + priv_s.sum() + priv_g.sum()).backward()
+    assert pool.stacked_private.w_up.grad is not None
+    assert float(pool.stacked_private.w_up.grad.float().abs().sum()) == 0.0

@@ -54,7 +54,7 @@ def test_argument_checks_fail_before_any_launch():
     assert lib.nestor_hip_path_mix_fwd(null, null, null, null, 1, 4, 12, null) == -22  # dim % 8
     assert lib.nestor_hip_path_mix_bwd(null, null, null, null, null, null, null, 7, 4, 16, null) == -22  # dtype
     assert lib.nestor_hip_path_scale_fwd(null, null, 2, null, null, 1, 4, 2, 2, 16, null) == -22  # which
-    assert lib.nestor_hip_path_scale_fwd(null, null, 1, null, null, 1, 4, 2, 8, 16, null) == -22  # no dest: widths differ
+    assert lib.nestor_hip_path_scale_fwd(null, null, 1, null, null, 1, 4, 2, 8, 16, null) == -22  # null operands
     assert lib.nestor_hip_path_scale_bwd(null, null, null, 1, null, null, null, 1, 4, 65, 65, 16, null) == -22  # slots > 64
     assert lib.nestor_hip_bias_rows_fwd(null, null, null, null, 0, null, 4, 12, null) == -22
     assert lib.nestor_hip_segment_colsum(null, null, null, null, null, 0, null, 4, 16, null) == -22  # splits
