@@ -773,19 +773,28 @@ __global__ __launch_bounds__(kRowBlock) void dispatch_scatter_kernel(
   const int lane = threadIdx.x % kWave;
   const int chunks = static_cast<int>(dim / 8);
   const uint16_t* src = x + t * dim;
-  for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
-    u32x4 v[kBatch];
-#pragma unroll
-    for (int b = 0; b < kBatch; ++b)
-      if (c0 + b * kWave < chunks) v[b] = ld16(src + (c0 + b * kWave) * 8);
-    for (int j = 0; j < slots; ++j) {
-      const int64_t p = row_dest[t * slots + j];
-      if (p < 0 || p >= rows_pad || !load_valid(pad_valid, p, valid_dtype) || pad_token[p] != t)
-        continue;
-      uint16_t* dst = out + p * dim;
+  // Lane j looks up assignment j (all of the token's map entries in one round of
+  // memory latency); the wavefront then walks the assignments that own a row.
+  for (int j0 = 0; j0 < slots; j0 += kWave) {
+    int64_t p = -1;
+    bool own = false;
+    if (j0 + lane < slots) {
+      p = row_dest[t * slots + j0 + lane];
+      own = p >= 0 && p < rows_pad && load_valid(pad_valid, p, valid_dtype) && pad_token[p] == t;
+    }
+    const uint64_t owners = __ballot(own);
+    for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
+      u32x4 v[kBatch];
 #pragma unroll
       for (int b = 0; b < kBatch; ++b)
-        if (c0 + b * kWave < chunks) st16(dst + (c0 + b * kWave) * 8, v[b]);
+        if (c0 + b * kWave < chunks) v[b] = ld16(src + (c0 + b * kWave) * 8);
+      for (uint64_t todo = owners; todo != 0; todo &= todo - 1) {
+        const int j = __ffsll(static_cast<long long>(todo)) - 1;
+        uint16_t* dst = out + __shfl(p, j, kWave) * dim;
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b)
+          if (c0 + b * kWave < chunks) st16(dst + (c0 + b * kWave) * 8, v[b]);
+      }
     }
   }
 }
