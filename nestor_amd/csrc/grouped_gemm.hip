@@ -18,11 +18,21 @@
 // indices for one output index -- the MFMA operand layout, with no transpose
 // pass over the weights or activations in HBM.
 //
-// Software pipeline per K step: the tile for step t+1 goes from registers to
-// the idle LDS buffer, the global loads for step t+2 are issued, then step t is
-// computed from the other buffer with MFMA operand fragments double-buffered in
-// registers, so global latency hides behind a whole K step and LDS latency
-// behind the previous fragment's MFMAs.
+// Four kernel families share these building blocks (in file order):
+//  * grouped_gemm_kernel -- register-staged: global -> registers -> padded LDS.
+//    Per K step the tile for step t+1 goes from registers to the idle LDS
+//    buffer, the global loads for step t+2 are issued, then step t is computed
+//    from the other buffer with MFMA operand fragments double-buffered in
+//    registers.  Takes any K that is a multiple of 8 and narrow outputs; the
+//    general fallback.
+//  * grouped_gemm_dma_kernel -- the row-tiled modes on the direct-to-LDS path
+//    (global_load_lds_dwordx4 into a three-stage unpadded ring, conflicts avoided
+//    by swizzling which 16-byte piece each lane fetches): the default at the
+//    measured shapes.
+//  * fp8w_stream_kernel -- e4m3 weights at a few rows per bank: the weight bytes
+//    stream through the same kind of ring, two workgroups per CU.
+//  * wgrad_persistent_kernel -- the weight gradient: one workgroup per CU walks a
+//    list of output tiles with the ring running across tile boundaries.
 //
 // The MFMA is issued with its operands swapped (B fragment first), which
 // produces the transposed 32 x 32 tile: every lane then holds four consecutive
