@@ -16,8 +16,16 @@ Pinning status (what independently fixes each function; see
   (brute force) and by reducing to the dropless plan when nothing overflows.
 * ``rows.*``                  -- per-row Python loops; finite differences in
   fp64 for the backward formulas; ``F.silu`` / ``torch.cat`` library routines.
+  The pool epilogues (``path_mix``, ``path_scale``) and the packed-attention
+  epilogue (``gate_combine_slots``) against element loops with hand-placed
+  roundings, their backward forms against fp64 autograd of the definition.
 * ``bank.segment_mm`` etc.    -- per-expert dense ``matmul`` (the reference's
-  own CPU fallback), the sparse per-expert loop, and a per-token loop.
+  own CPU fallback), the sparse per-expert loop, and a per-token loop; the
+  biased / pointwise gold against per-token ``F.linear`` on the per-expert
+  ``weight`` views.
 * ``router.*``                -- ``softmax`` / ``topk`` library routines on
-  tie-free inputs, top-1 renorm gate == 1, per-router loop for the batched form.
+  tie-free inputs, top-1 renorm gate == 1, per-router loop for the batched form;
+  the balancing step against a counting loop.
+
+No function of the oracle is "parity unpinned".
 """
