@@ -643,6 +643,19 @@ __device__ __forceinline__ void dma16(const void* src, uint32_t lds_addr) {
                : "s"(lds_addr), "v"(src)
                : "memory", "m0");
 }
+// The same with the source split into a wavefront-uniform base (scalar registers)
+// and a per-lane 32-bit byte offset: one address register per lane instead of
+// two, and the base advances with scalar arithmetic shared by all of a K step's
+// instructions instead of a 64-bit vector add per instruction.
+// The LDS destination is lds_base (scalar register) + kLdsOff (immediate), formed
+// in m0 by the one scalar add.
+template <int kLdsOff>
+__device__ __forceinline__ void dma16s(const void* base, uint32_t byte_off, uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_base), "v"(byte_off), "s"(base), "n"(kLdsOff)
+               : "memory", "m0", "scc");
+}
 __device__ __forceinline__ uint32_t lds_byte_addr(const void* p) {
   return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((NESTOR_LDS const void*)p));
 }
@@ -759,9 +772,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   const int kt_per_phase = static_cast<int>(p.K / BK);
   const int num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
 
-  // Per-lane source offsets (elements) of every DMA instruction, relative to a
-  // wavefront-uniform base that advances with the K step.
-  int64_t offa[C::A_CHUNKS], offb[C::B_CHUNKS];
+  // Per-lane byte offsets of every DMA instruction relative to a wavefront-uniform
+  // base that advances with the K step (and carries the row / bank origin).
+  uint32_t offa[C::A_CHUNKS], offb[C::B_CHUNKS];
   const int last_row = nrows - 1;
 #pragma unroll
   for (int i = 0; i < C::A_CHUNKS; ++i) {
@@ -770,8 +783,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     int row = ci / cpr;
     const int c = (ci % cpr) ^ ((row / rp) % cpr);
     row = row < last_row ? row : last_row;
-    offa[i] = static_cast<int64_t>(row0 + row) * p.lda + c * 8;
+    offa[i] = static_cast<uint32_t>((static_cast<int64_t>(row) * p.lda + c * 8) * 2);
   }
+  // Column origin of the tile: folded into the scalar base when it is in range for
+  // every lane, else (last column tile of a ragged width) clamped per lane.
 #pragma unroll
   for (int i = 0; i < C::B_CHUNKS; ++i) {
     const int blk = wave + kWaves * i;
@@ -782,7 +797,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       const int c = (ci % cpr) ^ ((row / rp) % cpr);
       int64_t n = n0 + row;
       n = n < p.N ? n : p.N - 1;
-      offb[i] = n * p.ldb + c * 8;
+      offb[i] = static_cast<uint32_t>(((n - n0) * p.ldb + c * 8) * 2);
     } else {
       // sub-tile s = which half of the instructions; inside it [BK][BW]
       constexpr int kPerSub = BK * BW / 8;  // pieces per sub-tile
@@ -791,39 +806,47 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       const int c = (cs % (BW / 8)) ^ (4 * (k & 3));
       int64_t n = n0 + c * 8;
       n = n < p.N ? n : p.N - 8;
-      offb[i] = static_cast<int64_t>(k) * p.ldb + n;
+      offb[i] = static_cast<uint32_t>((static_cast<int64_t>(k) * p.ldb + (n - n0)) * 2);
     }
   }
+  const uint16_t* a_origin = p.a + static_cast<int64_t>(row0) * p.lda;
+  const int64_t b_origin = bank * p.bank_stride + (kBContig ? n0 * p.ldb : n0);
 
   // DMA instruction q (A pieces first, then B pieces) of K step kt into ring
   // stage `stage`.  Steps past the end re-fetch the last step: the extra tile
   // lands in a stage nobody reads again, and every step then issues the same
   // number of instructions, which keeps the vmcnt bookkeeping uniform.
-  auto issue_one = [&](int kt, int stage, int q) __attribute__((always_inline)) {
+  // Byte offsets of a K step fit 32 bits (checked on the host): the step's scalar
+  // base is one 32-bit multiply and a 64-bit add, shared by the step's instructions.
+  const uint32_t a_step = BK * 2;
+  const uint32_t b_step = static_cast<uint32_t>(kBContig ? BK * 2 : BK * 2 * p.ldb);
+  const char* a_bytes = reinterpret_cast<const char*>(a_origin);
+  const char* b0_bytes = reinterpret_cast<const char*>(reinterpret_cast<const uint16_t*>(p.b0) + b_origin);
+  const char* b1_bytes = reinterpret_cast<const char*>(reinterpret_cast<const uint16_t*>(p.b1) + b_origin);
+  const uint32_t wave_lds = lds_byte_addr(lds) + wave * 1024;
+  auto issue_one = [&](int kt, int stage, auto q_tag) __attribute__((always_inline)) {
+    constexpr int q = decltype(q_tag)::value;
     kt = kt < num_kt ? kt : num_kt - 1;
-    uint16_t* sa = lds + stage * kStageElems;
-    uint16_t* sb = sa + C::A_ELEMS;
-    if (q < C::A_CHUNKS) {
-      const int i = q;
-      const uint16_t* src = p.a + offa[i] + static_cast<int64_t>(kt) * BK;
-      dma16(src, lds_byte_addr(sa + (wave + kWaves * i) * 512));
+    const uint32_t stage_lds = wave_lds + stage * (kStageElems * 2);
+    if constexpr (q < C::A_CHUNKS) {
+      dma16s<q * kWaves * 1024>(a_bytes + static_cast<uint32_t>(kt) * a_step, offa[q], stage_lds);
     } else {
-      const int i = q - C::A_CHUNKS;
-      const int blk = wave + kWaves * i;
-      const uint16_t* src;
+      constexpr int i = q - C::A_CHUNKS;
+      constexpr int kLdsOff = C::A_ELEMS * 2 + i * kWaves * 1024;
+      const char* base;
       if constexpr (kBContig) {
         const int phase = (kMode == kNTUpGate && kt >= kt_per_phase) ? 1 : 0;
-        const uint16_t* b = reinterpret_cast<const uint16_t*>(phase == 0 ? p.b0 : p.b1) +
-                            bank * p.bank_stride;
-        src = b + offb[i] + static_cast<int64_t>(kt - phase * kt_per_phase) * BK;
+        base = (phase == 0 ? b0_bytes : b1_bytes) +
+               static_cast<uint32_t>(kt - phase * kt_per_phase) * b_step;
       } else {
+        // blocks of the second sub-tile (the gate bank) are the upper half of the
+        // instructions: wave + kWaves * i >= kBlkPerSub for every wavefront
         constexpr int kBlkPerSub = BK * BW / 8 / 64;
-        const uint16_t* b =
-            reinterpret_cast<const uint16_t*>((kSub == 2 && blk >= kBlkPerSub) ? p.b1 : p.b0) +
-            bank * p.bank_stride;
-        src = b + offb[i] + static_cast<int64_t>(kt) * BK * p.ldb;
+        static_assert(kSub == 1 || kBlkPerSub % kWaves == 0, "a sub-tile is whole instructions");
+        constexpr bool kSecond = kSub == 2 && i * kWaves >= kBlkPerSub;
+        base = (kSecond ? b1_bytes : b0_bytes) + static_cast<uint32_t>(kt) * b_step;
       }
-      dma16(src, lds_byte_addr(sb + blk * 512));
+      dma16s<kLdsOff>(base, offb[i], stage_lds);
     }
   };
 
@@ -878,7 +901,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   // average half empty, and with one row of wavefronts per tile every
   // wavefront skips the same blocks).
   auto mfma_block = [&](auto mi_tag, int par, auto reads_tag, const uint16_t* ra, const uint16_t* rb,
-                        int rkk, int lt, int ls, int l0) __attribute__((always_inline)) {
+                        int rkk, int lt, int ls, auto l0_tag) __attribute__((always_inline)) {
     constexpr int kMi = decltype(mi_tag)::value;
     constexpr bool kDoReads = decltype(reads_tag)::value;
     constexpr int kMfmaEff = kMi * C::NJ, kReadsEff = kMi + C::NJ;
@@ -889,9 +912,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
         for (int r = m * kReadsEff / kMfmaEff; r < (m + 1) * kReadsEff / kMfmaEff; ++r)
           read_one(ra, rb, rkk, r, par ^ 1, kMi);
       }
-#pragma unroll
-      for (int q = m * kLoadsPerBlock / kMfmaEff; q < (m + 1) * kLoadsPerBlock / kMfmaEff; ++q)
-        issue_one(lt, ls, l0 + q);
+      constexpr int kQ0 = m * kLoadsPerBlock / kMfmaEff, kQ1 = (m + 1) * kLoadsPerBlock / kMfmaEff;
+      static_for<kQ1 - kQ0>([&](auto qc) __attribute__((always_inline)) {
+        issue_one(lt, ls, std::integral_constant<int, decltype(l0_tag)::value + kQ0 + decltype(qc)::value>{});
+      });
       constexpr int j = m / kMi, i = m % kMi;
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[par][j], fa[par][i], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
@@ -911,10 +935,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     const uint16_t* sb = sa + C::A_ELEMS;
     const uint16_t* na = lds + nxt * kStageElems;
     const uint16_t* nb = na + C::A_ELEMS;
-#pragma unroll
-    for (int kk = 0; kk + 1 < C::KK; ++kk)
+    static_for<C::KK - 1>([&](auto kc) __attribute__((always_inline)) {
+      constexpr int kk = decltype(kc)::value;
       mfma_block(mi_tag, kk & 1, std::true_type{}, sa, sb, kk + 1, kt + S - 1, prv,
-                 (kk + 1) * kLoadsPerBlock);
+                 std::integral_constant<int, (kk + 1) * kLoadsPerBlock>{});
+    });
     if constexpr (kNext) {
       // Step kt+1 has landed once only the later steps' instructions are
       // outstanding: steps kt+2 .. kt+S-1, all issued in full by now.
@@ -922,9 +947,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      mfma_block(mi_tag, (C::KK - 1) & 1, std::true_type{}, na, nb, 0, kt + S, cur, 0);
+      mfma_block(mi_tag, (C::KK - 1) & 1, std::true_type{}, na, nb, 0, kt + S, cur,
+                 std::integral_constant<int, 0>{});
     } else {
-      mfma_block(mi_tag, (C::KK - 1) & 1, std::false_type{}, na, nb, 0, kt + S, cur, 0);
+      mfma_block(mi_tag, (C::KK - 1) & 1, std::false_type{}, na, nb, 0, kt + S, cur,
+                 std::integral_constant<int, 0>{});
     }
   };
 
@@ -943,8 +970,7 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   if (num_kt > 0) {
 #pragma unroll
     for (int t = 0; t < S; ++t)
-#pragma unroll
-      for (int q = 0; q < kLoads; ++q) issue_one(t, t, q);
+      static_for<kLoads>([&](auto qc) __attribute__((always_inline)) { issue_one(t, t, qc); });
     wait_vmcnt<(S - 1) * kLoads>();
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -1626,7 +1652,11 @@ int dispatch_rows_gemm(const GemmParams& p, void* stream) {
     if (cfg == 3 && !(width >= 512 && p.K % 32 == 0)) cfg = 2;
   }
   if constexpr (kMode != kNNFp8W) {
-    // Direct-to-LDS variants: whole K steps only.
+    // Direct-to-LDS variants: whole K steps only, and byte offsets inside one bank's
+    // operand (and inside a tile's rows of activations) that fit 32 bits.
+    const bool b_contig = kMode == kNT || kMode == kNTUpGate;
+    const int64_t b_span = (b_contig ? p.N : p.K) * p.ldb * 2;
+    if (b_span >= (int64_t{1} << 32) || 512 * p.lda * 2 >= (int64_t{1} << 32)) cfg = 2;
     if (cfg == 3 && width >= 512 && p.K % 32 == 0) return launch_rows_dma<DmaXWide, kMode>(p, stream);
     if (cfg == 4 && width >= 256 && p.K % 64 == 0) return launch_rows_dma<DmaWide, kMode>(p, stream);
   }
