@@ -12,6 +12,13 @@
  *   - Index maps are int64 and segment ends (`offs`) int32, the widths the
  *     reference plan uses (nestor/backbones/grouped_mm.py:197-219,272-277).
  *   - Row-major tensors; a "bank" is one expert of a stacked weight tensor.
+ *   - Index tensors are read on the device and cannot be checked by the host
+ *     side of a call.  Bank ids, top-k choices and column selections are
+ *     clamped into their range by the kernels that read them (a bad value
+ *     gives a wrong result, not an access outside the tensors); row maps
+ *     (row_dest, pad_token, slot_rows, gid, ...) are taken as produced by
+ *     nestor_hip_index_build / nestor_hip_build_dispatch_maps and must index
+ *     inside the tensors they address.
  *
  * Each declaration cites the reference interface it stands in for (paths are
  * relative to the reference checkout).

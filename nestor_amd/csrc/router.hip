@@ -168,7 +168,9 @@ __global__ __launch_bounds__(kSlotsBlock) void private_slots_fwd_kernel(
   for (int j = 0; j < k_a; ++j) {
     int g;
     if (selected_in != nullptr) {
-      g = static_cast<int>(selected_in[t * k_a + j]);
+      // indices handed in are clamped into range: a bad one reads a wrong gate, never other memory
+      const int64_t given = selected_in[t * k_a + j];
+      g = static_cast<int>(given < 0 ? 0 : (given >= num_columns ? num_columns - 1 : given));
     } else {
       float best = -__builtin_inff();
       g = 0;
@@ -187,7 +189,8 @@ __global__ __launch_bounds__(kSlotsBlock) void private_slots_fwd_kernel(
     selected[t * k_a + j] = g;
     const float cg = load_scalar(column_gates, t * num_columns + g, dt);
     for (int i = 0; i < k_q; ++i) {
-      const int64_t e = choices[(t * num_columns + g) * k_q + i];
+      int64_t e = choices[(t * num_columns + g) * k_q + i];
+      e = e < 0 ? 0 : (e >= num_experts ? num_experts - 1 : e);
       const float pg = load_scalar(gates, (t * num_columns + g) * num_experts + e, dt);
       const int64_t slot = (t * k_a + j) * k_q + i;
       ids[slot] = static_cast<int64_t>(g) * num_experts + e;
@@ -226,11 +229,13 @@ __global__ __launch_bounds__(kSlotsBlock) void private_slots_bwd_kernel(
   for (int c = 0; c < num_columns * num_experts; ++c)
     store(grad_gates, t * num_columns * num_experts + c, 0.0f);
   for (int j = 0; j < k_a; ++j) {
-    const int64_t g = selected[t * k_a + j];
+    int64_t g = selected[t * k_a + j];
+    g = g < 0 ? 0 : (g >= num_columns ? num_columns - 1 : g);  // as the forward clamps them
     const float cg = load_scalar(column_gates, t * num_columns + g, dt);
     float dcg = 0.0f;
     for (int i = 0; i < k_q; ++i) {
-      const int64_t e = choices[(t * num_columns + g) * k_q + i];
+      int64_t e = choices[(t * num_columns + g) * k_q + i];
+      e = e < 0 ? 0 : (e >= num_experts ? num_experts - 1 : e);
       const float pg = load_scalar(gates, (t * num_columns + g) * num_experts + e, dt);
       const float dw = load_scalar(grad_weights, (t * k_a + j) * k_q + i, dt);
       const float term = dw * pg;

@@ -479,7 +479,9 @@ __global__ __launch_bounds__(kRowBlock) void path_scale_bwd_kernel(
   float dot = 0.0f;
   for (int s = 0; s < slots; ++s) {
     const int64_t o = dest == nullptr ? s : dest[t * slots + s];
-    const int64_t gbase = (t * num_out + o) * dim;
+    // a stream outside [0, num_out) selects nothing in the forward: zero gradient
+    const bool in_range = o >= 0 && o < num_out;
+    const int64_t gbase = (t * num_out + (in_range ? o : 0)) * dim;
     const int64_t ibase = (t * slots + s) * dim;
     for (int c0 = lane; c0 < chunks; c0 += kWave * kBatch) {
       float go[kBatch][8], v[kBatch][8];
@@ -489,6 +491,10 @@ __global__ __launch_bounds__(kRowBlock) void path_scale_bwd_kernel(
         if (c < chunks) {
           load8_as_f32<kF32>(g, gbase + c * 8, go[b]);
           load8_as_f32<kF32>(in, ibase + c * 8, v[b]);
+          if (!in_range) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) go[b][i] = 0.0f;
+          }
         }
       }
 #pragma unroll
