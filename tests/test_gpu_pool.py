@@ -130,3 +130,39 @@ def test_pool_on_an_empty_sequence_slice(cuda):
     (update.sum() + priv_s.sum() + priv_g.sum()).backward()
     assert pool.stacked_private.w_up.grad is not None
     assert float(pool.stacked_private.w_up.grad.float().abs().sum()) == 0.0
+
+
+def test_pool_under_checkpoint_recompute_and_on_sequence_slices(cuda):
+    """The reference runs the pool under activation-checkpoint recompute and on slices of
+    the sequence (nestor/backbones/nestor.py:9135-9153).  Recompute replays the forward
+    in the backward pass: outputs and every gradient must be bit-identical to the plain
+    run (the kernels are deterministic, no float atomics).  A call on the whole sequence
+    must equal the calls on its halves put together (tokens are independent)."""
+
+    from torch.utils.checkpoint import checkpoint
+
+    x, valid, gates, active, _ = _inputs(cuda)
+
+    def run(use_checkpoint):
+        pool = _pool(cuda, True).train()
+        xi = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            if use_checkpoint:
+                out = checkpoint(lambda a: pool(a, valid, gates, active)[0], xi, use_reentrant=False)
+            else:
+                out = pool(xi, valid, gates, active)[0]
+        out.float().square().sum().backward()
+        return out.detach(), xi.grad, {n: p.grad for n, p in pool.named_parameters()}
+
+    out0, gx0, gp0 = run(False)
+    out1, gx1, gp1 = run(True)
+    assert torch.equal(out0, out1) and torch.equal(gx0, gx1)
+    for n in gp0:
+        assert torch.equal(gp0[n], gp1[n]), n
+
+    pool = _pool(cuda, True)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        whole = pool(x, valid, gates, active)[0]
+        parts = [pool(x[:, a:b], valid[:, a:b], gates[:, a:b], active[:, a:b])[0]
+                 for a, b in ((0, 33), (33, 70))]
+    assert torch.equal(torch.cat(parts, dim=1), whole)
