@@ -26,7 +26,7 @@ sys.path.insert(0, ROOT)
 
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
-UPGATE_KERNEL_NAME = ("grouped_gemm_dma_kernel<DmaCfg<128,512,32,1,4,3>, kNNUpGate> "
+UPGATE_KERNEL_NAME = ("grouped_gemm_dma_kernel<DmaCfg<160,512,32,1,4,3>, kNNUpGate> "
                       "(private bank up|gate + SwiGLU)")
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "upgate_mlp_1b_hbm_counters.md")
 # the sources the dominant kernel is compiled from (the kernels and their shared header)
@@ -102,7 +102,7 @@ def kernel_breakdown(w, tensors, routed, iters: int = 5) -> dict:
 
     import ctypes
 
-    from nestor_amd import _lib, ops
+    from nestor_amd import ops, probes
     from nestor_amd.dispatch import dispatch_plan
 
     dev = tensors.x.device
@@ -126,23 +126,22 @@ def kernel_breakdown(w, tensors, routed, iters: int = 5) -> dict:
             entry.update(gbs=round(gbs, 1), frac_hbm_peak=round(gbs / HBM_PEAK_GBS, 4))
         out[name] = entry
 
-    wall_khz = _lib.load().nestor_hip_wall_clock_khz()
+    wall_khz = probes.wall_clock_khz()
 
     def shader_clock(name, fn):
         """Shader clock the chip holds during this GEMM, from the kernel's own
         counters (cycle counter against the constant-rate wall clock, summed over
-        its workgroups), and shader cycles per K step of a workgroup."""
+        its workgroups), and shader cycles per K step of a workgroup: three launches
+        of the measurement library's instrumented build of the same kernel source
+        (the product library carries no such hook)."""
         if wall_khz <= 0:
             return
         sink = torch.zeros(64, 4, dtype=torch.int64, device=dev)
         torch.cuda.synchronize()
-        _lib.call("nestor_hip_gemm_clock_sink", ctypes.c_void_p(sink.data_ptr()))
-        try:
+        with probes.instrumented(sink.data_ptr()):
             for _ in range(3):
                 fn()
             torch.cuda.synchronize()
-        finally:
-            _lib.call("nestor_hip_gemm_clock_sink", ctypes.c_void_p(0))
         cycles, ticks, _groups, steps = (int(v) for v in sink.sum(0).tolist())
         if ticks > 0 and steps > 0:
             out[name]["shader_mhz"] = round(cycles / ticks * wall_khz / 1000.0)
@@ -235,9 +234,9 @@ def mfma_clock_probe(dev, iters: int = 100000) -> dict:
 
     import ctypes
 
-    from nestor_amd import _lib
+    from nestor_amd import probes as _lib
 
-    wall_khz = _lib.load().nestor_hip_wall_clock_khz()
+    wall_khz = _lib.wall_clock_khz()
     out = {"instruction": "v_mfma_f32_32x32x16_bf16, 16 independent accumulator tiles per wavefront"}
     counters = torch.zeros(4, dtype=torch.int64, device=dev)
     for name, random_operands in (("constant_operands", 0), ("random_operands", 1)):
@@ -261,7 +260,8 @@ def mfma_clock_probe(dev, iters: int = 100000) -> dict:
     for reads, transfers in ((16, 0), (0, 8), (16, 8), (16, 10), (16, 12)):
         def run():
             _lib.call("nestor_hip_mfma_mix_probe", reads, transfers, rounds,
-                      ctypes.c_void_p(src.data_ptr()), region, ctypes.c_void_p(counters.data_ptr()),
+                      ctypes.c_void_p(src.data_ptr()), src.numel(), region,
+                      ctypes.c_void_p(counters.data_ptr()),
                       torch.cuda.current_stream().cuda_stream)
         ms = _event_ms(run, 3)
         cycles, ticks, instructions, _ = (int(v) for v in counters.tolist())
@@ -289,7 +289,8 @@ def traffic_probe(w, tensors, routed) -> None:
 
     import ctypes
 
-    from nestor_amd import _lib, ops
+    from nestor_amd import ops
+    from nestor_amd import probes as _lib
     from nestor_amd.dispatch import dispatch_plan
 
     dev = tensors.x.device
@@ -303,7 +304,7 @@ def traffic_probe(w, tensors, routed) -> None:
     rows = buf.numel() * 2 // row_bytes
     torch.cuda.synchronize()
     for piece, along_rows in ((512, 1), (64, 0), (1024, 1), (128, 0)):
-        _lib.call("nestor_hip_dma_stream_probe", ctypes.c_void_p(buf.data_ptr()), rows, row_bytes,
+        _lib.call("nestor_hip_dma_stream_probe", ctypes.c_void_p(buf.data_ptr()), buf.numel() * 2, rows, row_bytes,
                   piece, along_rows, stream)
         torch.cuda.synchronize()
     del buf

@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 14
+#define NESTOR_HIP_ABI_VERSION 15
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -85,13 +85,14 @@ const char* nestor_hip_strerror(int code);
  * nrows[cap] | count: tile t covers rows [row0[t], row0[t] + nrows[t]) of bank[t],
  * never crossing a segment end; bank == -1 marks a tile that lies wholly in the
  * slack tail behind the last segment (outputs are zero-filled, no product is
- * formed).  Three tables sit back to back: (1) every segment in tiles of up to
- * NESTOR_HIP_TILE_M = 128 rows, cap = max_tiles; (2) the same rows for the
- * kernels with 256-row tiles: the full 256-row tiles of each segment, plus its
- * remainder when that exceeds 128 rows, cap = rows_pad / 256 + num_banks + 2;
- * (3) the remainders of 1..128 rows that (2) leaves out, cap = num_banks + 2.
- * (1) alone, or (2) and (3) together, cover every row exactly once.  max_tiles
- * must equal nestor_hip_max_tiles(rows_pad, num_banks).
+ * formed).  Three tables sit back to back, each covering every row exactly once:
+ * (1) every segment in tiles of up to NESTOR_HIP_TILE_M = 128 rows, cap =
+ * max_tiles; (2) every segment in the fewest tiles of at most five 32-row blocks,
+ * the segment's blocks dealt evenly over them (a segment of 530 rows becomes tiles
+ * of 4, 4, 4 and 5 blocks instead of four full tiles and a fifth of 18 rows), cap =
+ * max_tiles; (3) the same with at most ten blocks per tile, cap = rows_pad / 256 +
+ * num_banks + 2.  The slack tail is cut at 128 / 160 / 320 rows.  max_tiles must
+ * equal nestor_hip_max_tiles(rows_pad, num_banks).
  * ---------------------------------------------------------------------- */
 size_t nestor_hip_index_build_workspace_bytes(int64_t rows, int32_t num_banks);
 int64_t nestor_hip_max_tiles(int64_t rows_pad, int32_t num_banks);
@@ -454,59 +455,6 @@ int nestor_hip_gate_slots_bwd(
     const int64_t* gid, const float* gates, const int64_t* slot_packed,
     void* grad_out_c /* bf16 [rows, dim] */, float* grad_gates /* nullable */,
     int64_t rows, int64_t dim, void* stream);
-
-/* ------------------------------------------------------------------------
- * Measurement aid (no counterpart in the reference): a stream of LDS-DMA
- * transfers over `rows` x `row_bytes` bytes at `src`, every byte fetched exactly
- * once, with the request shapes of the grouped GEMMs' operand fetches -- 1 KiB
- * per instruction as 1024 / piece_bytes consecutive rows x piece_bytes (64 ... 1024)
- * contiguous bytes, each wavefront walking along its rows (along_rows = 0) or down
- * its columns (along_rows = 1).  Run under `rocprofv3 --pmc FETCH_SIZE` it tells
- * how that counter prices such requests, which a plain copy kernel does not.
- * row_bytes % piece_bytes == 0 and rows % (1024 / piece_bytes) == 0.
- * ---------------------------------------------------------------------- */
-int nestor_hip_dma_stream_probe(
-    const void* src, int64_t rows, int64_t row_bytes, int32_t piece_bytes, int32_t along_rows,
-    void* stream);
-
-/* ------------------------------------------------------------------------
- * Measurement aids for the shader clock (no counterpart in the reference).  The
- * published matrix-core peak assumes the nominal clock; under a GEMM's load the
- * power management holds a lower one, and no profiler counter shows it.  A kernel
- * can: the ratio of its shader cycle counter to the constant-rate wall clock
- * (nestor_hip_wall_clock_khz ticks per millisecond) is the clock it ran at.
- *
- * nestor_hip_mfma_clock_probe: one workgroup per CU, four wavefronts each, issue
- * v_mfma_f32_32x32x16_bf16 back to back on 16 independent accumulator tiles with
- * no memory traffic, `iters` rounds; operands constant (random_operands = 0) or
- * random.  counters (device, 4 x uint64, the last one scratch) receives workgroup
- * 0's {shader cycles, wall-clock ticks} and the number of matrix instructions the
- * launch issued (each 2 * 32 * 32 * 16 flops); the caller times the launch.
- *
- * nestor_hip_gemm_clock_sink: from this call on the direct-to-LDS grouped-GEMM
- * kernels (row-tiled and weight-gradient) add, per workgroup, {shader cycles, wall
- * ticks, 1, K steps} to slot (workgroup index % 64) of sink (device, 64 x 4 uint64,
- * zeroed by the caller); NULL switches the hook off again.  Process-wide, not
- * synchronised with launches in flight: set it between synchronisations.
- * ---------------------------------------------------------------------- */
-int nestor_hip_mfma_clock_probe(int32_t random_operands, int32_t iters, uint64_t* counters,
-                                void* stream);
-/* The main loop of the GEMM kernels and nothing around it: a wavefront multiplies a
- * 128 x 128 accumulator tile in blocks of 16 MFMAs on fragments it read from LDS during
- * the block before (random bf16 values, two register sets), with reads_per_step 1 KiB
- * fragment reads and transfers_per_step 1 KiB LDS-DMA transfers per K step of 32 MFMAs
- * between the matrix instructions at the kernels' spacing -- no barriers, no waiting for
- * the transfers' data, no epilogue, no tile switches, every transfer an L2 hit (the
- * workgroups of an XCD share region_bytes of src, which holds 8 regions; region_bytes a
- * multiple of 32 KiB, at least 64 KiB).  Supported (reads, transfers): (0,0) (16,0) (0,8)
- * (16,8) (16,10) (16,12) -- 16/8 is the mix of the 256 x 256 x 32 kernels, 16/10 that of
- * the 128 x 512 x 32 ones with both operands read as whole fragments.  One round is 32
- * MFMAs; counters as above. */
-int nestor_hip_mfma_mix_probe(int32_t reads_per_step, int32_t transfers_per_step, int32_t iters,
-                              const void* src, int64_t region_bytes, uint64_t* counters,
-                              void* stream);
-int nestor_hip_wall_clock_khz(void); /* ticks of wall_clock64() per millisecond; < 0 on error */
-int nestor_hip_gemm_clock_sink(uint64_t* sink);
 
 #ifdef __cplusplus
 }

@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_int32, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libnestor_hip.so"
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 F32 = 0
 BF16 = 1
@@ -92,11 +92,6 @@ _SIGNATURES: dict[str, list] = {
     "nestor_hip_path_scale_bwd": [
         _P, _P, _P, _I32, _P, _P, _P, _I32, _I64, _I32, _I32, _I64, _P,
     ],
-    "nestor_hip_dma_stream_probe": [_P, _I64, _I64, _I32, _I32, _P],
-    "nestor_hip_mfma_clock_probe": [_I32, _I32, _P, _P],
-    "nestor_hip_mfma_mix_probe": [_I32, _I32, _I32, _P, _I64, _P, _P],
-    "nestor_hip_wall_clock_khz": [],
-    "nestor_hip_gemm_clock_sink": [_P],
 }
 _RESTYPES = {
     "nestor_hip_strerror": c_char_p,

@@ -130,12 +130,20 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // The three tile tables of a tile_table buffer (written by the index build, walked by
 // the grouped GEMMs): their capacities depend on the static sizes only.
-enum TileKind { kTiles128 = 0, kTiles256 = 1, kTilesRest = 2 };
+//   kTiles128     every segment cut into tiles of up to 128 rows;
+//   kTilesBal160  every segment cut into the fewest tiles of up to five 32-row blocks,
+//                 the blocks dealt evenly over a segment's tiles;
+//   kTilesBal320  the same with up to ten 32-row blocks per tile.
+enum TileKind { kTiles128 = 0, kTilesBal160 = 1, kTilesBal320 = 2, kTileKinds = 3 };
 
+// 32-row blocks a tile of this kind holds at most.
+__host__ __device__ inline int tile_blocks_cap(int kind) {
+  return kind == kTiles128 ? 4 : kind == kTilesBal160 ? 5 : 10;
+}
+// A balanced table never holds more tiles than cutting at 128 (256) rows would.
 __host__ __device__ inline int64_t table_cap(int kind, int64_t rows_pad, int num_banks) {
-  if (kind == kTiles128) return rows_pad / 128 + num_banks + 2;
-  if (kind == kTiles256) return rows_pad / 256 + num_banks + 2;
-  return num_banks + 2;
+  if (kind == kTilesBal320) return rows_pad / 256 + num_banks + 2;
+  return rows_pad / 128 + num_banks + 2;
 }
 __host__ __device__ inline int64_t table_offset(int kind, int64_t rows_pad, int num_banks) {
   int64_t off = 0;

@@ -8,6 +8,7 @@
 #include <utility>
 
 #include "common.hpp"
+#include "dma_addressing.hpp"
 
 namespace nestor {
 
@@ -15,6 +16,12 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 
 #define NESTOR_LDS __attribute__((address_space(3)))
+
+// Instrumented build (the measurement library only): the direct-to-LDS kernels add their
+// cycle and wall-clock counts to a caller-provided sink.  Compiled out of the product.
+#ifndef NESTOR_GEMM_CLOCK_HOOK
+#define NESTOR_GEMM_CLOCK_HOOK 0
+#endif
 
 // Output tiles are written once and read by a later kernel.
 #ifndef NESTOR_GEMM_NT_STORES
@@ -173,6 +180,9 @@ __device__ __forceinline__ void interleave_memory(std::integer_sequence<int, Ms.
 }
 
 // Tile configuration of the direct-to-LDS kernels (ring of STAGES_ unpadded stages).
+// BM is the tallest tile the configuration takes; a wavefront holds up to MI = BM / WGM /
+// 32 row blocks of 32 x WTN accumulators (the fifth block, where there is one, in
+// ordinary vector registers: the accumulation registers hold four).
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int STAGES_, int OCC_ = 1>
 struct DmaCfg {
   static constexpr int OCC = OCC_;  // workgroups resident per CU the register budget is sized for
@@ -180,20 +190,26 @@ struct DmaCfg {
   static constexpr int WAVES = WGM * WGN, THREADS = 64 * WAVES;
   static_assert(WAVES == 4 || WAVES == 8, "one or two wavefronts per SIMD");
   static constexpr int WTM = BM / WGM, WTN = BN / WGN;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "whole MFMA tiles");
   static constexpr int MI = WTM / 32, NJ = WTN / 32;
+  static_assert(MI >= 1 && MI <= 5, "four row blocks in accumulation registers, a fifth in vector registers");
   static constexpr int KK = BK / 16;
-  static constexpr int STAGE_LD = BN + 8;
-  static constexpr int A_ELEMS = BM * BK, B_ELEMS = BN * BK;
-  static constexpr int STAGE_ELEMS = BM * STAGE_LD;
+  // Rows of the A stage: BM rounded up to whole transfer instructions per wavefront.
+  static constexpr int A_ROW_UNIT = THREADS * 8 / BK;
+  static constexpr int A_ROWS = (BM + A_ROW_UNIT - 1) / A_ROW_UNIT * A_ROW_UNIT;
+  static constexpr int A_ELEMS = A_ROWS * BK, B_ELEMS = BN * BK;
   static constexpr int kStages = STAGES_;
   static constexpr int PIPE_ELEMS = kStages * (A_ELEMS + B_ELEMS);
+  // Epilogue: one slab of 32 rows x WTN columns per wavefront, inside the drained ring.
+  static constexpr int EPI_LD = WTN + 8;
+  static constexpr int EPI_ELEMS = WAVES * 32 * EPI_LD;
   static constexpr size_t LDS_BYTES =
-      sizeof(uint16_t) * (PIPE_ELEMS > STAGE_ELEMS ? PIPE_ELEMS : STAGE_ELEMS);
-  static constexpr int A_CHUNKS = BM * BK / 8 / THREADS;  // DMA instructions per lane
+      sizeof(uint16_t) * (PIPE_ELEMS > EPI_ELEMS ? PIPE_ELEMS : EPI_ELEMS);
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS of one CU");
+  static constexpr int A_CHUNKS = A_ROWS * BK / 8 / THREADS;  // DMA instructions per lane
   static constexpr int B_CHUNKS = BN * BK / 8 / THREADS;
-  static_assert(BM * BK / 8 % THREADS == 0 && BN * BK / 8 % THREADS == 0, "chunking");
+  static_assert(BN * BK / 8 % THREADS == 0, "chunking");
   static_assert(KK % 2 == 0, "fragment double-buffer parity");
-  static_assert((A_CHUNKS + B_CHUNKS) % KK == 0, "DMA instructions split evenly over the MFMA blocks");
 };
 
 // One LDS-DMA instruction: 64 lanes x 16 bytes from per-lane global addresses to

@@ -478,8 +478,30 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(GemmParams p) {
 // piece c ^ f(row); a contraction-major tile XORs the 32-byte column block with
 // the low bits of its row.  Fragment reads apply the same XOR.
 //
+// Tiles are as tall as their table entry says, up to C::BM rows: a wavefront
+// multiplies mi = ceil(ceil(rows / 32) / WGM) of its C::MI row blocks (the same
+// count in every wavefront row) and the wavefront rows sit 32 * mi rows apart, so
+// a tile of 96 or of 160 rows costs its own blocks and nothing else.  The balanced
+// tile tables use that: a segment's 32-row blocks are dealt evenly over the fewest
+// tiles instead of leaving a short last tile that would stream a whole weight panel
+// for a few rows.  Four row blocks accumulate in the accumulation registers; a
+// fifth (C::MI == 5) accumulates in ordinary vector registers through the
+// vector-register form of the MFMA, issued as inline assembly (the compiler
+// only ever picks one register class for all of a kernel's MFMAs).
+//
 // Requirement checked by the launcher: the contraction length is a multiple of
 // BK.  Row-tiled modes only; the weight gradient has its own kernel below.
+// A-stage transfer instructions per lane that a tile of mi row blocks per wavefront row
+// needs: its 32 * mi * WGM rows, in whole instructions.
+template <typename C>
+constexpr int a_chunks_needed(int mi) {
+  return (32 * mi * C::WGM + C::A_ROW_UNIT - 1) / C::A_ROW_UNIT;
+}
+
+__device__ __forceinline__ void mfma_vgpr(f32x16& c, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+
 template <typename C, int kMode>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(GemmParams p) {
   static_assert(kMode != kTN && kMode != kNNFp8W, "row-tiled bf16 modes");
@@ -490,11 +512,15 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   constexpr bool kBContig = kMode == kNT || kMode == kNTUpGate;
   constexpr int kOutCols = kUpGateFwd ? BN / 2 : BN;
   // The forward up|gate tile is two contraction-major sub-tiles side by side
-  // (up columns, gate columns) so that one DMA instruction reads one bank.
+  // (up columns, gate columns) so that one DMA instruction reads one bank.  A
+  // wavefront multiplies WTN / 2 columns of the up sub-tile and the same columns of
+  // the gate sub-tile, so each lane ends up with matching up and gate values.
   constexpr int kSub = kUpGateFwd ? 2 : 1;
   constexpr int BW = BN / kSub;
+  static_assert(!kUpGateFwd || (C::NJ % 2 == 0), "half of a wavefront's column blocks are up, half gate");
   constexpr int kStageElems = C::A_ELEMS + C::B_ELEMS;
-  constexpr int kLoads = C::A_CHUNKS + C::B_CHUNKS;
+  constexpr int kAccMi = C::MI < 4 ? C::MI : 4;  // row blocks held in accumulation registers
+  constexpr bool kAgprReads = kAccMi * C::NJ == 16;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront-uniform: keep it scalar
@@ -503,12 +529,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
 
   // Workgroup b runs on XCD b % 8.  For the GEMMs with few column tiles and a
   // long contraction (down projection, fused up|gate input gradient) each XCD
-  // takes groups of four consecutive row tiles (about one expert at 512 rows per
-  // expert) with all their column tiles, so the tiles that share an activation
-  // panel and the tiles that share a weight panel meet in the same L2 (measured
-  // +3..5 %).  The GEMMs that stream wide weight panels once do better when all
-  // XCDs walk the same expert at the same time, each on its own column tiles
-  // (plain order, column tile fastest).
+  // takes groups of consecutive row tiles with all their column tiles, so the
+  // tiles that share an activation panel and the tiles that share a weight panel
+  // meet in the same L2.  The GEMMs that stream wide weight panels once do as well
+  // when all XCDs walk the same expert at the same time, each on its own column
+  // tiles (plain order, column tile fastest).
   int tile, nt;
   if (p.tile_group > 0) {
     const int xcd = blockIdx.x & 7;
@@ -525,6 +550,14 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       tile = (group * 8 + xcd) * p.tile_group + within % p.tile_group;
       nt = within / p.tile_group;
     }
+  } else if (p.tile_order == 2) {
+    // every XCD keeps n_tiles / 8 ADJACENT column tiles of every row tile (the launcher
+    // checks that n_tiles is a multiple of 8): with column tiles dealt x, x + 8, ... the
+    // XCDs with the even ones ran 6 % longer than the others and the launch waited for them
+    const int per = p.n_tiles >> 3;
+    const int seq = blockIdx.x >> 3;
+    tile = seq / per;
+    nt = (blockIdx.x & 7) * per + seq % per;
   } else {
     tile = blockIdx.x / p.n_tiles;
     nt = blockIdx.x % p.n_tiles;
@@ -533,7 +566,8 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   if (tile >= tt[3 * p.max_tiles]) return;
   const int bank = tt[tile];
   const int row0 = tt[p.max_tiles + tile];
-  const int nrows = tt[2 * p.max_tiles + tile];
+  int nrows = tt[2 * p.max_tiles + tile];
+  nrows = nrows < BM ? nrows : BM;  // the launcher pairs every configuration with a table it covers
   const int64_t n0 = static_cast<int64_t>(nt) * kOutCols;
   if (bank < 0) {
     const u32x4 zero = {0, 0, 0, 0};
@@ -558,48 +592,36 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
 
   const int kt_per_phase = static_cast<int>(p.K / BK);
   const int num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
+#if NESTOR_GEMM_CLOCK_HOOK
   unsigned long long clk_c0 = 0, clk_w0 = 0;
   if (p.clock_sink != nullptr) {
     clk_c0 = clock64();
     clk_w0 = wall_clock64();
   }
+#endif
+
+  // Row blocks per wavefront in this tile, and where this wavefront's rows start.
+  int mi_eff = (((nrows + 31) >> 5) + C::WGM - 1) / C::WGM;
+  mi_eff = mi_eff < 1 ? 1 : (mi_eff > C::MI ? C::MI : mi_eff);
+  mi_eff = __builtin_amdgcn_readfirstlane(mi_eff);
+  const int wave_row0 = 32 * mi_eff * wm;
 
   // Per-lane byte offsets of every DMA instruction relative to a wavefront-uniform
-  // base that advances with the K step (and carries the row / bank origin).
+  // base that advances with the K step (and carries the row / bank origin).  Rows
+  // behind the tile's last one (also the rows that only round the A stage up to
+  // whole instructions) fetch the last row again: what they feed is never stored.
   uint32_t offa[C::A_CHUNKS], offb[C::B_CHUNKS];
   const int last_row = nrows - 1;
 #pragma unroll
-  for (int i = 0; i < C::A_CHUNKS; ++i) {
-    const int ci = (wave + kWaves * i) * 64 + lane;  // 16-byte position in the tile
-    constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
-    int row = ci / cpr;
-    const int c = (ci % cpr) ^ ((row / rp) % cpr);
-    row = row < last_row ? row : last_row;
-    offa[i] = static_cast<uint32_t>((static_cast<int64_t>(row) * p.lda + c * 8) * 2);
-  }
-  // Column origin of the tile: folded into the scalar base when it is in range for
-  // every lane, else (last column tile of a ragged width) clamped per lane.
+  for (int i = 0; i < C::A_CHUNKS; ++i)
+    offa[i] = dma::a_lane_offset<BK>((wave + kWaves * i) * 64 + lane, last_row, p.lda);
+  // Column origin of the tile: part of the scalar base; the last column tile of a ragged
+  // width is clamped per lane.
 #pragma unroll
   for (int i = 0; i < C::B_CHUNKS; ++i) {
-    const int blk = wave + kWaves * i;
-    const int ci = blk * 64 + lane;
-    if constexpr (kBContig) {
-      constexpr int cpr = BK / 8, rp = 256 / (BK * 2);
-      const int row = ci / cpr;
-      const int c = (ci % cpr) ^ ((row / rp) % cpr);
-      int64_t n = n0 + row;
-      n = n < p.N ? n : p.N - 1;
-      offb[i] = static_cast<uint32_t>(((n - n0) * p.ldb + c * 8) * 2);
-    } else {
-      // sub-tile s = which half of the instructions; inside it [BK][BW]
-      constexpr int kPerSub = BK * BW / 8;  // pieces per sub-tile
-      const int cs = ci % kPerSub;
-      const int k = cs / (BW / 8);
-      const int c = (cs % (BW / 8)) ^ (4 * (k & 3));
-      int64_t n = n0 + c * 8;
-      n = n < p.N ? n : p.N - 8;
-      offb[i] = static_cast<uint32_t>((static_cast<int64_t>(k) * p.ldb + (n - n0)) * 2);
-    }
+    const int ci = (wave + kWaves * i) * 64 + lane;
+    if constexpr (kBContig) offb[i] = dma::b_contig_lane_offset<BK>(ci, n0, p.N, p.ldb);
+    else offb[i] = dma::b_major_lane_offset<BK, BW>(ci, n0, p.N, p.ldb);
   }
   const uint16_t* a_origin = p.a + static_cast<int64_t>(row0) * p.lda;
   const int64_t b_origin = bank * p.bank_stride + (kBContig ? n0 * p.ldb : n0);
@@ -616,14 +638,17 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   const char* b0_bytes = reinterpret_cast<const char*>(reinterpret_cast<const uint16_t*>(p.b0) + b_origin);
   const char* b1_bytes = reinterpret_cast<const char*>(reinterpret_cast<const uint16_t*>(p.b1) + b_origin);
   const uint32_t wave_lds = lds_byte_addr(lds) + wave * 1024;
-  auto issue_one = [&](int kt, int stage, auto q_tag) __attribute__((always_inline)) {
+  // a_tag: how many A instructions per lane the tile's height needs (the rows behind
+  // 32 * mi * WGM are never read, so a short tile does not fetch them).
+  auto issue_one = [&](int kt, int stage, auto a_tag, auto q_tag) __attribute__((always_inline)) {
+    constexpr int kA = decltype(a_tag)::value;
     constexpr int q = decltype(q_tag)::value;
     kt = kt < num_kt ? kt : num_kt - 1;
     const uint32_t stage_lds = wave_lds + stage * (kStageElems * 2);
-    if constexpr (q < C::A_CHUNKS) {
+    if constexpr (q < kA) {
       dma16s<q * kWaves * 1024>(a_bytes + static_cast<uint32_t>(kt) * a_step, offa[q], stage_lds);
     } else {
-      constexpr int i = q - C::A_CHUNKS;
+      constexpr int i = q - kA;
       constexpr int kLdsOff = C::A_ELEMS * 2 + i * kWaves * 1024;
       const char* base;
       if constexpr (kBContig) {
@@ -642,9 +667,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     }
   };
 
-  f32x16 acc[C::MI][C::NJ];
+  f32x16 acc[kAccMi][C::NJ];
+  f32x16 accv[C::NJ];  // the fifth row block (C::MI == 5 only)
 #pragma unroll
-  for (int i = 0; i < C::MI; ++i)
+  for (int i = 0; i < kAccMi; ++i)
 #pragma unroll
     for (int j = 0; j < C::NJ; ++j)
 #pragma unroll
@@ -653,23 +679,27 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   const int kc_row = lane & 31, kc_piece = lane >> 5;
   const int tr_krow = 8 * (lane >> 5) + ((lane & 15) >> 2);
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int a_wave_elems = wave_row0 * BK;  // this wavefront's first row inside an A stage
   // Fragment read r of a fragment set into the registers of parity `par`, in
   // the order the MFMAs consume them: B fragment 0, the A fragments, then the
   // remaining B fragments.
   bf16x8 fa[2][C::MI], fb[2][C::NJ];
-  auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par, int mi_eff) __attribute__((always_inline)) {
-    if (r >= 1 && r <= mi_eff) {
+  auto read_one = [&](const uint16_t* sa, const uint16_t* sb, int kk, int r, int par, int mi_n) __attribute__((always_inline)) {
+    if (r >= 1 && r <= mi_n) {
       const int i = r - 1;
-      const int row = C::WTM * wm + 32 * i + kc_row;
-      fa[par][i] = *reinterpret_cast<const bf16x8*>(sa + kc_offset<BK>(row, 2 * kk + kc_piece));
+      // wave_row0 is a multiple of 32 rows: the swizzle of a row depends on its low bits only
+      fa[par][i] = *reinterpret_cast<const bf16x8*>(sa + a_wave_elems +
+                                                    kc_offset<BK>(32 * i + kc_row, 2 * kk + kc_piece));
     } else {
-      const int j = r == 0 ? 0 : r - mi_eff;
+      const int j = r == 0 ? 0 : r - mi_n;
       if constexpr (kBContig) {
         const int row = C::WTN * wn + 32 * j + kc_row;
         fb[par][j] = *reinterpret_cast<const bf16x8*>(sb + kc_offset<BK>(row, 2 * kk + kc_piece));
       } else {
-        const int col = C::WTN * wn + 32 * j;      // column inside the B tile
-        const uint16_t* sub = sb + (col / BW) * (BK * BW);
+        // column inside the B tile: its sub-tile, and the column inside that
+        const int half = kUpGateFwd ? j / (C::NJ / 2) : 0;
+        const int col = kUpGateFwd ? (C::WTN / 2) * wn + 32 * (j % (C::NJ / 2)) : C::WTN * wn + 32 * j;
+        const uint16_t* sub = sb + (kUpGateFwd ? half : col / BW) * (BK * BW);
         const int k = 16 * kk + tr_krow;
         const int n = (col % BW) + tr_col;
         fb[par][j] = lds_read_tr_pair<BW>(sub + nc_offset<BW>(k, n));
@@ -677,26 +707,27 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     }
   };
 
-  constexpr int kReads = C::MI + C::NJ;   // fragments per set
-  constexpr int kMfma = C::MI * C::NJ;
-  constexpr int kLoadsPerBlock = kLoads / C::KK;
   constexpr int S = C::kStages;
 
   // One block of MFMAs on the fragment set of parity `par`, with this block's
   // share of the memory instructions placed between them in program order:
-  // the reads of the next fragment set (into parity par ^ 1) and kLoadsPerBlock
-  // DMA instructions starting at number l0 of K step lt.  The scheduling
-  // barriers pin that order: memory instructions issued in a burst back up the
-  // address path and stall the wavefront's matrix instructions behind them.
+  // the reads of the next fragment set (into parity par ^ 1) and share `share_tag`
+  // of the DMA instructions of K step lt (a step's instructions are dealt over its KK
+  // blocks: share s is [s * kLoads / KK, (s + 1) * kLoads / KK)).  The scheduling barriers pin that order:
+  // memory instructions issued in a burst back up the address path and stall the
+  // wavefront's matrix instructions behind them.
   // mi_tag: how many of the wavefront's 32-row blocks hold rows of the tile; the
-  // MFMAs and A fragments of the others are skipped (a segment's last tile is on
-  // average half empty, and with one row of wavefronts per tile every
-  // wavefront skips the same blocks).
+  // MFMAs and A fragments of the others are skipped.
   auto mfma_block = [&](auto mi_tag, int par, auto reads_tag, const uint16_t* ra, const uint16_t* rb,
-                        int rkk, int lt, int ls, auto l0_tag) __attribute__((always_inline)) {
+                        int rkk, int lt, int ls, auto share_tag) __attribute__((always_inline)) {
     constexpr int kMi = decltype(mi_tag)::value;
     constexpr bool kDoReads = decltype(reads_tag)::value;
     constexpr int kMfmaEff = kMi * C::NJ, kReadsEff = kMi + C::NJ;
+    using ATag = std::integral_constant<int, a_chunks_needed<C>(kMi)>;
+    constexpr int kLoads = ATag::value + C::B_CHUNKS;
+    constexpr int kShare = decltype(share_tag)::value;
+    constexpr int kL0 = kShare * kLoads / C::KK;
+    constexpr int kLn = (kShare + 1) * kLoads / C::KK - kL0;
     static_for<kMfmaEff>([&](auto mc) __attribute__((always_inline)) {
       constexpr int m = decltype(mc)::value;
       if constexpr (kDoReads) {
@@ -704,12 +735,16 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
         for (int r = m * kReadsEff / kMfmaEff; r < (m + 1) * kReadsEff / kMfmaEff; ++r)
           read_one(ra, rb, rkk, r, par ^ 1, kMi);
       }
-      constexpr int kQ0 = m * kLoadsPerBlock / kMfmaEff, kQ1 = (m + 1) * kLoadsPerBlock / kMfmaEff;
+      constexpr int kQ0 = m * kLn / kMfmaEff, kQ1 = (m + 1) * kLn / kMfmaEff;
       static_for<kQ1 - kQ0>([&](auto qc) __attribute__((always_inline)) {
-        issue_one(lt, ls, std::integral_constant<int, decltype(l0_tag)::value + kQ0 + decltype(qc)::value>{});
+        issue_one(lt, ls, ATag{}, std::integral_constant<int, kL0 + kQ0 + decltype(qc)::value>{});
       });
       constexpr int j = m / kMi, i = m % kMi;
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[par][j], fa[par][i], acc[i][j], 0, 0, 0);
+      if constexpr (i < 4) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[par][j], fa[par][i], acc[i][j], 0, 0, 0);
+      } else {
+        mfma_vgpr(accv[j], fb[par][j], fa[par][i]);
+      }
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -727,10 +762,11 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     const uint16_t* sb = sa + C::A_ELEMS;
     const uint16_t* na = lds + nxt * kStageElems;
     const uint16_t* nb = na + C::A_ELEMS;
+    constexpr int kLoads = a_chunks_needed<C>(decltype(mi_tag)::value) + C::B_CHUNKS;
     static_for<C::KK - 1>([&](auto kc) __attribute__((always_inline)) {
       constexpr int kk = decltype(kc)::value;
       mfma_block(mi_tag, kk & 1, std::true_type{}, sa, sb, kk + 1, kt + S - 1, prv,
-                 std::integral_constant<int, (kk + 1) * kLoadsPerBlock>{});
+                 std::integral_constant<int, kk + 1>{});
     });
     if constexpr (kNext) {
       // Step kt+1 has landed once only the later steps' instructions are
@@ -749,6 +785,20 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
 
   auto k_loop = [&](auto mi_tag) __attribute__((always_inline)) {
     constexpr int kMi = decltype(mi_tag)::value;
+    using ATag = std::integral_constant<int, a_chunks_needed<C>(kMi)>;
+    constexpr int kLoads = ATag::value + C::B_CHUNKS;
+#pragma unroll
+    for (int t = 0; t < S; ++t)
+      static_for<kLoads>([&](auto qc) __attribute__((always_inline)) { issue_one(t, t, ATag{}, qc); });
+    if constexpr (kMi == 5) {
+#pragma unroll
+      for (int j = 0; j < C::NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) accv[j][e] = 0.0f;
+    }
+    wait_vmcnt<(S - 1) * kLoads>();
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int r = 0; r < kMi + C::NJ; ++r) read_one(lds, lds + C::A_ELEMS, 0, r, 0, kMi);
     int cur = 0;
@@ -757,94 +807,122 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       cur = cur == S - 1 ? 0 : cur + 1;
     }
     k_step(mi_tag, num_kt - 1, cur, std::false_type{});
+    if constexpr (kMi == 5) {
+      // The fifth block's MFMAs are opaque to the compiler's hazard bookkeeping: keep the
+      // epilogue's first read of their results behind the matrix pipe's write-back.
+      asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+    }
   };
 
   if (num_kt > 0) {
-#pragma unroll
-    for (int t = 0; t < S; ++t)
-      static_for<kLoads>([&](auto qc) __attribute__((always_inline)) { issue_one(t, t, qc); });
-    wait_vmcnt<(S - 1) * kLoads>();
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    // Row blocks in use: only tiles with a single row of wavefronts can skip.
-    int mi_eff = C::MI;
-    if constexpr (C::WGM == 1 && C::MI == 4) {
-      mi_eff = (nrows + 31) >> 5;
-      mi_eff = mi_eff < 1 ? 1 : (mi_eff > 4 ? 4 : mi_eff);
-    }
-    if constexpr (C::WGM == 1 && C::MI == 4) {
-      switch (mi_eff) {
-        case 1: k_loop(std::integral_constant<int, 1>{}); break;
-        case 2: k_loop(std::integral_constant<int, 2>{}); break;
-        case 3: k_loop(std::integral_constant<int, 3>{}); break;
-        default: k_loop(std::integral_constant<int, 4>{}); break;
-      }
-    } else {
-      k_loop(std::integral_constant<int, C::MI>{});
+    switch (mi_eff) {
+      case 1: k_loop(std::integral_constant<int, 1>{}); break;
+      case 2:
+        if constexpr (C::MI >= 2) k_loop(std::integral_constant<int, 2>{});
+        break;
+      case 3:
+        if constexpr (C::MI >= 3) k_loop(std::integral_constant<int, 3>{});
+        break;
+      case 4:
+        if constexpr (C::MI >= 4) k_loop(std::integral_constant<int, 4>{});
+        break;
+      default:
+        if constexpr (C::MI >= 5) k_loop(std::integral_constant<int, 5>{});
+        break;
     }
   }
   wait_vmcnt<0>();
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
 
-  // ---- epilogue (same as the register-staged kernel) -----------------------
-  uint16_t* stage = lds;
+  // ---- epilogue, per wavefront ----------------------------------------------
+  // The ring is drained and nobody reads it again: each wavefront takes a slab of
+  // 32 rows x WTN columns in it, writes one row block of its accumulators there as
+  // bf16, reads the block back row by row and stores whole 128- or 256-byte row
+  // pieces.  No workgroup barrier: the same wavefront wrote and reads, in program
+  // order.  Up and gate of a column sit in the same lane (see kSub above), so the
+  // fused SwiGLU needs nothing from another wavefront.
+  constexpr int kEpiLd = C::EPI_LD;
+  uint16_t* slab = lds + wave * (32 * kEpiLd);
+  const int col0 = kUpGateFwd ? (C::WTN / 2) * wn : C::WTN * wn;  // first output column in the tile
+  static_for<C::MI>([&](auto ic) __attribute__((always_inline)) {
+    constexpr int i = decltype(ic)::value;
+    const int rbase = wave_row0 + 32 * i;  // tile row of the block's first row
+    if (i < mi_eff && rbase < nrows) {
+      __builtin_amdgcn_sched_barrier(0);  // one slab's worth of registers at a time
 #pragma unroll
-  for (int i = 0; i < C::MI; ++i)
+      for (int j = 0; j < C::NJ; ++j)
 #pragma unroll
-    for (int j = 0; j < C::NJ; ++j)
+        for (int q = 0; q < 4; ++q) {
+          const int n = 32 * j + 8 * q + 4 * (lane >> 5);
+          float v[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int m = C::WTM * wm + 32 * i + (lane & 31);
-        const int n = C::WTN * wn + 32 * j + 8 * q + 4 * (lane >> 5);
-        float v[4];
+          for (int e = 0; e < 4; ++e) {
+            if constexpr (i >= 4) {
+              v[e] = accv[j][4 * q + e];
+            } else if constexpr (kAgprReads) {
+              // 256 accumulator registers live in AGPRs; reading them where they
+              // are used keeps the compiler from hoisting every read and spilling.
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][4 * q + e]));
+            } else {
+              v[e] = acc[i][j][4 * q + e];
+            }
+          }
+          u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          *reinterpret_cast<u32x2*>(slab + (lane & 31) * kEpiLd + n) = packed;
+        }
+      if constexpr (kUpGateFwd) {
+        constexpr int kHalf = C::WTN / 2;   // up columns of the slab, then the same gate columns
+        constexpr int kCpr = kHalf / 8;     // 16-byte pieces per row of either
+        constexpr int kPieces = 32 * kCpr / 64;
+        u32x4 up[kPieces], gate[kPieces];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if constexpr (C::MI * C::NJ == 16) {
-            // 256 accumulator registers live in AGPRs; reading them where they
-            // are used keeps the compiler from hoisting every read and spilling.
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][4 * q + e]));
-          } else {
-            v[e] = acc[i][j][4 * q + e];
+        for (int t = 0; t < kPieces; ++t) {
+          const int c = lane + 64 * t;
+          up[t] = *reinterpret_cast<const u32x4*>(slab + (c / kCpr) * kEpiLd + (c % kCpr) * 8);
+          gate[t] = *reinterpret_cast<const u32x4*>(slab + (c / kCpr) * kEpiLd + kHalf + (c % kCpr) * 8);
+        }
+#pragma unroll
+        for (int t = 0; t < kPieces; ++t) {
+          const int c = lane + 64 * t;
+          const int row = rbase + c / kCpr;
+          const int64_t n = n0 + col0 + (c % kCpr) * 8;
+          if (row < nrows && n < p.N) {
+            const int64_t r = row0 + row;
+            if (p.out != nullptr) {
+              st16o(p.out + r * p.ldo + n, up[t]);
+              st16o(p.out + r * p.ldo + p.N + n, gate[t]);
+            }
+            float u[8], g[8], h[8];
+            unpack8(up[t], u);
+            unpack8(gate[t], g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[e] = silu_rounded(g[e]) * u[e];
+            st16o(p.out2 + r * p.ldo2 + n, pack8(h));
           }
         }
-        u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        *reinterpret_cast<u32x2*>(stage + m * C::STAGE_LD + n) = packed;
-      }
-  __syncthreads();
-  if constexpr (kUpGateFwd) {
-    constexpr int kHalfChunks = BN / 16;
-    for (int c = tid; c < BM * kHalfChunks; c += kThreads) {
-      const int row = c / kHalfChunks;
-      const int hc = c % kHalfChunks;
-      const int64_t n = n0 + hc * 8;
-      if (row < nrows && n < p.N) {
-        const int64_t r = row0 + row;
-        const u32x4 up = *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + hc * 8);
-        const u32x4 gate =
-            *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + BN / 2 + hc * 8);
-        if (p.out != nullptr) {
-          st16o(p.out + r * p.ldo + n, up);
-          st16o(p.out + r * p.ldo + p.N + n, gate);
-        }
-        float u[8], g[8], h[8];
-        unpack8(up, u);
-        unpack8(gate, g);
+      } else {
+        constexpr int kCpr = C::WTN / 8;
+        constexpr int kPieces = 32 * kCpr / 64;
+        u32x4 piece[kPieces];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) h[e] = silu_rounded(g[e]) * u[e];
-        st16o(p.out2 + r * p.ldo2 + n, pack8(h));
+        for (int t = 0; t < kPieces; ++t) {
+          const int c = lane + 64 * t;
+          piece[t] = *reinterpret_cast<const u32x4*>(slab + (c / kCpr) * kEpiLd + (c % kCpr) * 8);
+        }
+#pragma unroll
+        for (int t = 0; t < kPieces; ++t) {
+          const int c = lane + 64 * t;
+          const int row = rbase + c / kCpr;
+          const int64_t n = n0 + col0 + (c % kCpr) * 8;
+          if (row < nrows && n < p.N) st16o(p.out + (row0 + row) * p.ldo + n, piece[t]);
+        }
       }
     }
-  } else {
-    for (int c = tid; c < BM * (BN / 8); c += kThreads) {
-      const int row = c / (BN / 8);
-      const int64_t n = n0 + (c % (BN / 8)) * 8;
-      if (row < nrows && n < p.N)
-        st16o(p.out + (row0 + row) * p.ldo + n,
-             *reinterpret_cast<const u32x4*>(stage + row * C::STAGE_LD + (c % (BN / 8)) * 8));
-    }
-  }
+  });
+#if NESTOR_GEMM_CLOCK_HOOK
   if (p.clock_sink != nullptr && tid == 0) clock_sink_add(p.clock_sink, clk_c0, clk_w0, num_kt);
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -945,11 +1023,13 @@ __global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmPar
   }
   __syncthreads();
   if (count == 0) return;
+#if NESTOR_GEMM_CLOCK_HOOK
   unsigned long long clk_c0 = 0, clk_w0 = 0, clk_steps = 0;
   if (p.clock_sink != nullptr) {
     clk_c0 = clock64();
     clk_w0 = wall_clock64();
   }
+#endif
   auto steps_of = [&](int i) __attribute__((always_inline)) -> int {
     const int4 t = table[i];
     return __builtin_amdgcn_readfirstlane((t.y - t.x + BK - 1) / BK);
@@ -971,17 +1051,9 @@ __global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmPar
   static_assert(BM / 8 == 32 && BN / 8 == 32, "one DMA instruction covers two contraction rows");
   uint32_t offa[C::A_CHUNKS], offb[C::B_CHUNKS];
 #pragma unroll
-  for (int c = 0; c < C::A_CHUNKS; ++c) {
-    const int krow = 2 * (wave + kWaves * c) + (lane >> 5);
-    const int pc = (lane & 31) ^ (4 * (krow & 3));
-    offa[c] = static_cast<uint32_t>((static_cast<int64_t>(krow) * p.lda + pc * 8) * 2);
-  }
+  for (int c = 0; c < C::A_CHUNKS; ++c) offa[c] = dma::wgrad_lane_offset(wave, kWaves, c, lane, p.lda);
 #pragma unroll
-  for (int c = 0; c < C::B_CHUNKS; ++c) {
-    const int krow = 2 * (wave + kWaves * c) + (lane >> 5);
-    const int pc = (lane & 31) ^ (4 * (krow & 3));
-    offb[c] = static_cast<uint32_t>((static_cast<int64_t>(krow) * p.ldb + pc * 8) * 2);
-  }
+  for (int c = 0; c < C::B_CHUNKS; ++c) offb[c] = dma::wgrad_lane_offset(wave, kWaves, c, lane, p.ldb);
   i32x4 desc_a = buffer_descriptor(p.a, 0), desc_b = buffer_descriptor(p.b0, 0);
   // bytes per K step; the launcher checks that a whole operand spans less than 4 GiB
   const uint32_t step_a = static_cast<uint32_t>(BK * p.lda * 2), step_b = static_cast<uint32_t>(BK * p.ldb * 2);
@@ -1012,14 +1084,11 @@ __global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmPar
     const int n0 = nt * BN;
     // valid bytes from the descriptor's base: whole rows up to the segment's last
     // one, of which the tile's own columns
-    const int cols_a = static_cast<int>(p.M) - m0 < BM ? static_cast<int>(p.M) - m0 : BM;
-    const int cols_b = static_cast<int>(p.N) - n0 < BN ? static_cast<int>(p.N) - n0 : BN;
-    desc_a = buffer_descriptor(
-        p.a + static_cast<int64_t>(beg) * p.lda + m0,
-        static_cast<uint32_t>((static_cast<int64_t>(seg_rows - 1) * p.lda + cols_a) * 2));
+    desc_a = buffer_descriptor(p.a + static_cast<int64_t>(beg) * p.lda + m0,
+                               dma::wgrad_num_records(seg_rows, p.lda, p.M, m0, BM));
     desc_b = buffer_descriptor(
         reinterpret_cast<const uint16_t*>(p.b0) + static_cast<int64_t>(beg) * p.ldb + n0,
-        static_cast<uint32_t>((static_cast<int64_t>(seg_rows - 1) * p.ldb + cols_b) * 2));
+        dma::wgrad_num_records(seg_rows, p.ldb, p.N, n0, BN));
     return true;
   };
   // DMA instruction q of the cursor's K step.
@@ -1277,10 +1346,14 @@ __global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmPar
       for (int kt = 1; kt < num_kt; ++kt) k_step(std::false_type{}, std::false_type{});
     }
     epilogue(item);
+#if NESTOR_GEMM_CLOCK_HOOK
     clk_steps += num_kt;
+#endif
   }
   wait_vmcnt<0>();
+#if NESTOR_GEMM_CLOCK_HOOK
   if (p.clock_sink != nullptr && tid == 0) clock_sink_add(p.clock_sink, clk_c0, clk_w0, clk_steps);
+#endif
 }
 
 // Tile configurations.  Row-tiled modes need BM == NESTOR_HIP_TILE_M.
@@ -1308,28 +1381,38 @@ int launch_rows(GemmParams p, void* stream) {
   return launch_status();
 }
 
-using DmaXWide = DmaCfg<128, 512, 32, 1, 4, 3>;   // wavefront tile 128 x 128, 3-stage DMA ring
-using DmaWide = DmaCfg<128, 256, 64, 2, 2, 3>;    // wavefront tile 64 x 128
+// Each configuration walks the tile table whose tiles it covers.
+using DmaXWide = DmaCfg<160, 512, 32, 1, 4, 3>;   // up to 5 row blocks x (128 x 128 per wavefront); balanced 160-row table
+using DmaSquare = DmaCfg<320, 256, 32, 2, 2, 3>;  // 2 x 2 wavefronts of up to 5 blocks x 128 columns; balanced 320-row table
+using DmaWide = DmaCfg<128, 256, 64, 2, 2, 3>;    // wavefront tile 64 x 128; 128-row table
 using WgradPers = DmaCfg<256, 256, 32, 2, 2, 3>;  // persistent weight gradient
-using DmaSquare = DmaCfg<256, 256, 32, 2, 2, 3>;  // 256-row tiles, wavefront tile 128 x 128
 
-// Measurement hook: where the direct-to-LDS kernels add their cycle and wall-clock
-// counts (see GemmParams::clock_sink); null unless nestor_hip_gemm_clock_sink set it.
+#if NESTOR_GEMM_CLOCK_HOOK
+// Measurement hook (instrumented build only): where the direct-to-LDS kernels add their
+// cycle and wall-clock counts (see GemmParams::clock_sink); null unless
+// nestor_hip_gemm_clock_sink set it.
 unsigned long long* g_clock_sink = nullptr;
+#endif
 
 template <typename C, int kMode>
-int launch_rows_dma(GemmParams p, void* stream) {
+int launch_rows_dma(GemmParams p, int table_kind, int64_t rows_pad, int32_t num_banks, void* stream) {
+  static_assert(C::BM == 128 || C::BM == 160 || C::BM == 320, "a tile table exists for these heights");
+  if (32 * tile_blocks_cap(table_kind) > C::BM) return NESTOR_HIP_EINVAL;
+  p.tile_table += table_offset(table_kind, rows_pad, num_banks);
+  p.max_tiles = table_cap(table_kind, rows_pad, num_banks);
   constexpr int out_cols = kMode == kNNUpGate ? C::BN / 2 : C::BN;
   p.n_tiles = static_cast<int>(ceil_div(p.N, out_cols));
+#if NESTOR_GEMM_CLOCK_HOOK
   p.clock_sink = g_clock_sink;
+#endif
   static const int forced_group = config_choice("NESTOR_HIP_TILE_GROUP", -1);
-  // Measured at the 1b-like shapes: the down projection runs best (and fetches least:
-  // 4.6 GB instead of 7.8 GB per launch) with eight row tiles per XCD group walked row
-  // tile first; the fused input gradient with four, column tile first; the others in
-  // plain order.  The spread is 2-3 %: none of these launches is bound by its traffic.
+  // Measured at the 1b-like shapes: the down projection runs best (and fetches least)
+  // with eight row tiles per XCD group walked row tile first; the fused input gradient
+  // with four, column tile first; the others in plain order.  The spread is 2-6 %.
   p.tile_group = forced_group >= 0 ? forced_group : (kMode == kNN ? 8 : kMode == kNTUpGate ? 4 : 0);
   static const int forced_order = config_choice("NESTOR_HIP_TILE_ORDER", -1);
   p.tile_order = forced_order >= 0 ? forced_order : (kMode == kNN ? 1 : 0);
+  if (p.tile_order == 2 && (p.tile_group > 0 || p.n_tiles % 8 != 0)) p.tile_order = 0;
   // whole groups of row tiles per XCD (see the kernel's tile mapping)
   const int64_t gran = p.tile_group > 0 ? 8 * p.tile_group : 1;
   const int64_t blocks = ceil_div(p.max_tiles, gran) * gran * p.n_tiles;
@@ -1346,7 +1429,7 @@ int launch_rows_dma(GemmParams p, void* stream) {
   return launch_status();
 }
 
-// Row-tiled modes: which kernel(s) walk which of the buffer's tile tables.
+// Row-tiled modes: which kernel walks which of the buffer's tile tables.
 template <int kMode>
 int dispatch_rows_gemm(const GemmParams& p, int64_t rows_pad, int32_t num_banks, void* stream) {
   static const int forced = config_choice("NESTOR_HIP_GEMM_CFG", -1);
@@ -1355,39 +1438,26 @@ int dispatch_rows_gemm(const GemmParams& p, int64_t rows_pad, int32_t num_banks,
   constexpr bool kBContigMode = kMode == kNT || kMode == kNTUpGate;
   if (cfg < 0) {
     // Measured on the 1b-like shapes: the direct-to-LDS variants win in every
-    // mode.  The forward GEMMs (weights contraction-major) prefer the 128x512x32
-    // tile.  The input-gradient GEMMs (both operands contraction-contiguous, so
-    // every transfer is made of 64-byte row pieces) prefer 256x256x32, which moves
-    // 20 % fewer pieces per MFMA: +9-10 % on segments that fill the tiles; they
-    // walk the 256-row table and finish each segment's remainder of up to 128 rows
-    // with the 128-row kernel (cfg 7).  Shapes these do not cover (narrow outputs,
-    // a contraction that is not a multiple of the K step) take the
-    // register-staged kernel.
+    // mode.  The forward GEMMs (weights contraction-major) prefer the x512x32 tile
+    // with one row of wavefronts (cfg 3).  The input-gradient GEMMs (both operands
+    // contraction-contiguous, so every transfer is made of 64-byte row pieces) prefer
+    // x256x32 with 2 x 2 wavefronts (cfg 7), which moves 20 % fewer pieces per MFMA.
+    // Narrower outputs take the x256x64 tile (cfg 4); a contraction that is not a
+    // multiple of the K step takes the register-staged kernel (cfg 2 and below).
     cfg = kBContigMode ? 7 : 3;
-    if (cfg == 7 && !(width >= 512 && p.K % 64 == 0)) cfg = kMode == kNTUpGate ? 4 : 3;
-    if (cfg == 4 && !(width >= 256 && p.K % 64 == 0)) cfg = 3;
-    if (cfg == 3 && !(width >= 512 && p.K % 32 == 0)) cfg = 2;
+    if (cfg == 3 && width < 512) cfg = 4;
   }
   if constexpr (kMode != kNNFp8W) {
     // Direct-to-LDS variants: whole K steps only, and byte offsets inside one bank's
     // operand (and inside a tile's rows of activations) that fit 32 bits.
     const int64_t b_span = (kBContigMode ? p.N : p.K) * p.ldb * 2;
-    if (b_span >= (int64_t{1} << 32) || 512 * p.lda * 2 >= (int64_t{1} << 32)) cfg = 2;
-    if (cfg == 7 && width >= 512 && p.K % 64 == 0) {
-      GemmParams big = p;
-      big.tile_table = p.tile_table + table_offset(kTiles256, rows_pad, num_banks);
-      big.max_tiles = table_cap(kTiles256, rows_pad, num_banks);
-      const int rc = launch_rows_dma<DmaSquare, kMode>(big, stream);
-      if (rc != NESTOR_HIP_OK) return rc;
-      GemmParams rest = p;
-      rest.tile_table = p.tile_table + table_offset(kTilesRest, rows_pad, num_banks);
-      rest.max_tiles = table_cap(kTilesRest, rows_pad, num_banks);
-      if constexpr (kMode == kNTUpGate) return launch_rows_dma<DmaWide, kMode>(rest, stream);
-      return launch_rows_dma<DmaXWide, kMode>(rest, stream);
-    }
-    if (cfg == 7) cfg = 3;
-    if (cfg == 3 && width >= 512 && p.K % 32 == 0) return launch_rows_dma<DmaXWide, kMode>(p, stream);
-    if (cfg == 4 && width >= 256 && p.K % 64 == 0) return launch_rows_dma<DmaWide, kMode>(p, stream);
+    const bool spans_fit = b_span < (int64_t{1} << 32) && 512 * p.lda * 2 < (int64_t{1} << 32);
+    if (spans_fit && cfg == 7 && width >= 256 && p.K % 32 == 0)
+      return launch_rows_dma<DmaSquare, kMode>(p, kTilesBal320, rows_pad, num_banks, stream);
+    if (spans_fit && (cfg == 3 || cfg == 7) && width >= 512 && p.K % 32 == 0)
+      return launch_rows_dma<DmaXWide, kMode>(p, kTilesBal160, rows_pad, num_banks, stream);
+    if (spans_fit && cfg >= 3 && width >= 256 && p.K % 64 == 0)
+      return launch_rows_dma<DmaWide, kMode>(p, kTiles128, rows_pad, num_banks, stream);
   }
   if (cfg >= 3) cfg = 2;
   if (cfg == 2 && width < 512) cfg = 1;
@@ -1571,7 +1641,9 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
     }
     const int64_t items = ceil_div(M, C::BM) * ceil_div(N, C::BN) * num_banks;
     if (num_cus >= 8 && items / num_cus + 2 <= WgradLayout<C>::kMaxItems) {
+#if NESTOR_GEMM_CLOCK_HOOK
       p.clock_sink = g_clock_sink;
+#endif
       if (p.out_f32)
         hipLaunchKernelGGL((wgrad_persistent_kernel<C, true>), dim3(static_cast<unsigned>(num_cus)),
                            dim3(C::THREADS), WgradLayout<C>::LDS_BYTES,
@@ -1591,7 +1663,9 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
   }
 }
 
+#if NESTOR_GEMM_CLOCK_HOOK
 extern "C" int nestor_hip_gemm_clock_sink(uint64_t* sink) {
   g_clock_sink = reinterpret_cast<unsigned long long*>(sink);
   return NESTOR_HIP_OK;
 }
+#endif

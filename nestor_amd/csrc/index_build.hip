@@ -177,20 +177,18 @@ __device__ __forceinline__ void zero_slot(int64_t p, int64_t* pad_token,
 // Tile tables.  A table is bank[cap] | row0[cap] | nrows[cap] | count for a capacity
 // `cap` fixed by the static sizes; three of them sit back to back in the tile_table
 // buffer:
-//   kTiles128   every segment cut into tiles of up to 128 rows, then the slack tail
-//               behind the last segment as bank == -1 tiles (the table the 128-row
-//               kernels walk);
-//   kTiles256   the same rows cut for the 256-row kernels: floor(len / 256) full tiles
-//               per segment plus one more when the remainder exceeds 128 rows, then
-//               the slack tail as bank == -1 tiles of up to 256 rows;
-//   kTilesRest  the remainders of 1..128 rows that kTiles256 leaves out, as 128-row
-//               tiles: one launch over kTiles256 and one over kTilesRest cover every
-//               row exactly once.
+//   kTiles128     every segment cut into tiles of up to 128 rows, then the slack tail
+//                 behind the last segment as bank == -1 tiles;
+//   kTilesBal160  every segment cut into the fewest tiles of at most five 32-row
+//                 blocks, its blocks dealt evenly over them (530 rows = 17 blocks ->
+//                 tiles of 4, 4, 4 and 5 blocks, not four full tiles and a fifth of 18
+//                 rows that streams a whole weight panel for them), then the slack tail;
+//   kTilesBal320  the same with at most ten blocks per tile (the 2 x 2 wavefront tiles).
+// Every table covers every padded row exactly once.
 __device__ __forceinline__ int tiles_of(int kind, int len) {
   if (kind == kTiles128) return (len + 127) / 128;
-  const int rem = len % 256;
-  if (kind == kTiles256) return len / 256 + (rem > 128 ? 1 : 0);
-  return rem > 0 && rem <= 128 ? 1 : 0;
+  const int cap = tile_blocks_cap(kind);
+  return ((len + 31) / 32 + cap - 1) / cap;
 }
 
 // Writes one table for segments [start[e], start[e] + len[e]) held in LDS.
@@ -199,7 +197,7 @@ __device__ __forceinline__ void emit_tiles(int kind, const int32_t* seg_start, c
                            int64_t tail_begin, int64_t tail_end, int32_t* tile_table,
                            int64_t max_tiles) {
   const int tid = threadIdx.x;
-  const int tile_rows = kind == kTiles256 ? 256 : 128;
+  const int tile_rows = 32 * tile_blocks_cap(kind);
   for (int e = tid; e < num_banks; e += kScanBlock) tile_first[e] = tiles_of(kind, seg_len[e]);
   __syncthreads();
   const int bank_tiles = block_exclusive_scan(tile_first, num_banks, scratch);
@@ -209,23 +207,31 @@ __device__ __forceinline__ void emit_tiles(int kind, const int32_t* seg_start, c
   // a wavefront per bank, a lane per tile: a single bank with hundreds of tiles (a whole
   // batch as one segment) and hundreds of banks with a few tiles each both stay short
   for (int e = tid / kWave; e < num_banks; e += kScanBlock / kWave) {
-    const int n = tiles_of(kind, seg_len[e]);
-    // the remainder table starts behind the full 256-row tiles of its segment
-    const int first_row = kind == kTilesRest ? seg_len[e] / 256 * 256 : 0;
+    const int len = seg_len[e];
+    const int n = tiles_of(kind, len);
+    const int64_t blocks = (len + 31) / 32;
     for (int j = tid % kWave; j < n; j += kWave) {
       const int64_t t = tile_first[e] + j;
       if (t < max_tiles) {
-        const int left = seg_len[e] - first_row - j * tile_rows;
+        // tile j of n takes blocks [j * blocks / n, (j + 1) * blocks / n); cutting at 128
+        // rows is the same rule with the blocks dealt four at a time
+        int first, rows;
+        if (kind == kTiles128) {
+          first = j * 128;
+          rows = 128;
+        } else {
+          const int b0 = static_cast<int>(j * blocks / n), b1 = static_cast<int>((j + 1) * blocks / n);
+          first = 32 * b0;
+          rows = 32 * (b1 - b0);
+        }
+        const int left = len - first;
         t_bank[t] = e;
-        t_row0[t] = seg_start[e] + first_row + j * tile_rows;
-        t_rows[t] = left < tile_rows ? left : tile_rows;
+        t_row0[t] = seg_start[e] + first;
+        t_rows[t] = left < rows ? left : rows;
       }
     }
   }
-  // The slack tail belongs to the first two tables (each covers all rows by itself
-  // or together with the remainder table).
-  const int64_t tail_tiles =
-      kind == kTilesRest ? 0 : (tail_end - tail_begin + tile_rows - 1) / tile_rows;
+  const int64_t tail_tiles = (tail_end - tail_begin + tile_rows - 1) / tile_rows;
   for (int64_t j = tid; j < tail_tiles; j += kScanBlock) {
     const int64_t t = bank_tiles + j;
     if (t < max_tiles) {
@@ -249,7 +255,7 @@ __device__ __forceinline__ void emit_all_tiles(const int32_t* seg_start, const i
                                int32_t* tile_first, int32_t* scratch, int num_banks,
                                int64_t tail_begin, int64_t tail_end, int64_t rows_pad,
                                int32_t* tile_table) {
-  for (int kind = 0; kind < 3; ++kind)
+  for (int kind = 0; kind < kTileKinds; ++kind)
     emit_tiles(kind, seg_start, seg_len, tile_first, scratch, num_banks, tail_begin, tail_end,
                tile_table + table_offset(kind, rows_pad, num_banks),
                table_cap(kind, rows_pad, num_banks));
@@ -541,7 +547,7 @@ extern "C" int64_t nestor_hip_max_tiles(int64_t rows_pad, int32_t num_banks) {
 }
 
 extern "C" int64_t nestor_hip_tile_table_ints(int64_t rows_pad, int32_t num_banks) {
-  return table_offset(3, rows_pad, num_banks);
+  return table_offset(kTileKinds, rows_pad, num_banks);
 }
 
 namespace nestor {

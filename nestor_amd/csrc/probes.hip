@@ -15,6 +15,7 @@
 // walks down the rows, like K steps over a contraction-major one).  Every byte of
 // the buffer is fetched exactly once.
 #include "common.hpp"
+#include "nestor_hip_probes.h"
 
 namespace nestor {
 namespace {
@@ -253,10 +254,12 @@ extern "C" int nestor_hip_wall_clock_khz(void) {
   return khz;
 }
 
-extern "C" int nestor_hip_dma_stream_probe(const void* src, int64_t rows, int64_t row_bytes,
-                                           int32_t piece_bytes, int32_t along_rows,
-                                           void* stream) {
+extern "C" int nestor_hip_dma_stream_probe(const void* src, int64_t src_bytes, int64_t rows,
+                                           int64_t row_bytes, int32_t piece_bytes,
+                                           int32_t along_rows, void* stream) {
   if (!src || rows <= 0 || row_bytes <= 0) return NESTOR_HIP_EINVAL;
+  // the walk touches exactly rows * row_bytes bytes from src on
+  if (rows > INT64_MAX / row_bytes || rows * row_bytes > src_bytes) return NESTOR_HIP_EINVAL;
   if (piece_bytes != 64 && piece_bytes != 128 && piece_bytes != 256 && piece_bytes != 512 &&
       piece_bytes != 1024)
     return NESTOR_HIP_EINVAL;
@@ -268,11 +271,13 @@ extern "C" int nestor_hip_dma_stream_probe(const void* src, int64_t rows, int64_
 }
 
 extern "C" int nestor_hip_mfma_mix_probe(int32_t reads_per_step, int32_t transfers_per_step,
-                                         int32_t iters, const void* src, int64_t region_bytes,
-                                         uint64_t* counters, void* stream) {
+                                         int32_t iters, const void* src, int64_t src_bytes,
+                                         int64_t region_bytes, uint64_t* counters, void* stream) {
   if (!counters || !src || iters <= 0) return NESTOR_HIP_EINVAL;
-  // every workgroup's walk stays inside its XCD's region: whole 4 KiB steps, 32 KiB starts
+  // every workgroup's walk stays inside its XCD's region: whole 4 KiB steps, 32 KiB starts;
+  // the eight regions lie back to back from src on
   if (region_bytes < 65536 || region_bytes % 32768 != 0) return NESTOR_HIP_EINVAL;
+  if (region_bytes > INT64_MAX / 8 || 8 * region_bytes > src_bytes) return NESTOR_HIP_EINVAL;
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)

@@ -53,10 +53,12 @@ def max_tiles_for(rows_pad: int, num_banks: int) -> int:
 
 
 def tile_table_ints(rows_pad: int, num_banks: int) -> int:
-    """int32 entries of a tile_table buffer: the 128-row table, the 256-row table and the
-    table of remainders, each ``3 * cap + 1`` (``nestor_hip_tile_table_ints``)."""
+    """int32 entries of a tile_table buffer: the 128-row table and the two balanced tables
+    (tiles of up to 160 and up to 320 rows), each ``3 * cap + 1``
+    (``nestor_hip_tile_table_ints``)."""
 
-    caps = (max_tiles_for(rows_pad, num_banks), rows_pad // 256 + num_banks + 2, num_banks + 2)
+    cap = max_tiles_for(rows_pad, num_banks)
+    caps = (cap, cap, rows_pad // 256 + num_banks + 2)
     return sum(3 * c + 1 for c in caps)
 
 

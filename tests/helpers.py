@@ -50,12 +50,14 @@ def zipf_ids(seed: int, num_tokens: int, slots: int, num_banks: int, alpha: floa
 
 def tile_tables(tile_table: torch.Tensor, rows_pad: int, num_banks: int):
     """The three tables of a tile_table buffer as ``(bank, row0, nrows)`` triples of their
-    live entries: 128-row tiles, 256-row tiles, remainders the 256-row table leaves out.
+    live entries: 128-row tiles, balanced tiles of up to 160 rows, balanced tiles of up to
+    320 rows.
     Also returns a copy of the buffer with every unspecified entry (beyond each table's
     count) zeroed, for bit-for-bit comparisons of two builds."""
 
     tt = tile_table.detach().cpu().clone()
-    caps = (rows_pad // 128 + num_banks + 2, rows_pad // 256 + num_banks + 2, num_banks + 2)
+    caps = (rows_pad // 128 + num_banks + 2, rows_pad // 128 + num_banks + 2,
+            rows_pad // 256 + num_banks + 2)
     assert tt.numel() == sum(3 * c + 1 for c in caps)
     out, base = [], 0
     for cap in caps:

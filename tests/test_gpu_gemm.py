@@ -134,11 +134,10 @@ def test_slack_tail_is_zero_filled(cuda):
 
 
 def test_clock_hook_counts_workgroups_and_leaves_results_alone(cuda):
-    """The measurement hook of the direct-to-LDS kernels: results are the same bits
-    with it on, it counts every workgroup that multiplied, and it stops when cleared."""
-    import ctypes
-
-    from nestor_amd import _lib, ops
+    """The instrumented GEMM build of the measurement library: the same bits as the
+    product kernels, every workgroup that multiplied is counted, and outside the
+    ``instrumented`` block the product library runs (it has no hook at all)."""
+    from nestor_amd import ops, probes
 
     tokens, slots, banks, K, N = 2048, 2, 8, 1024, 2048
     want, got = _setup(tokens, slots, banks, cuda)
@@ -149,8 +148,7 @@ def test_clock_hook_counts_workgroups_and_leaves_results_alone(cuda):
     plain_w = ops.grouped_gemm_tn(a, g, got.offs, got.padded_starts, got.counts)
     sink = torch.zeros(64, 4, dtype=torch.int64, device=cuda)
     torch.cuda.synchronize()
-    _lib.call("nestor_hip_gemm_clock_sink", ctypes.c_void_p(sink.data_ptr()))
-    try:
+    with probes.instrumented(sink.data_ptr()):
         hooked = ops.grouped_gemm_nn(a, b, got.tile_table)
         torch.cuda.synchronize()
         rows_total = sink.sum(0).tolist()
@@ -158,13 +156,12 @@ def test_clock_hook_counts_workgroups_and_leaves_results_alone(cuda):
         hooked_w = ops.grouped_gemm_tn(a, g, got.offs, got.padded_starts, got.counts)
         torch.cuda.synchronize()
         wgrad_total = sink.sum(0).tolist()
-    finally:
-        _lib.call("nestor_hip_gemm_clock_sink", ctypes.c_void_p(0))
     assert torch.equal(plain, hooked) and torch.equal(plain_w, hooked_w)
     for cycles, ticks, groups, steps in (rows_total, wgrad_total):
         assert cycles > 0 and ticks > 0 and groups > 0 and steps >= groups
-    # row-tiled launch: one workgroup per (row tile with rows, column tile of 512), K / 32 steps each
-    tiles = sum((int(c) + 127) // 128 for c in want.counts.tolist())
+    # row-tiled launch: one workgroup per (balanced row tile, column tile of 512), K / 32 steps each
+    padded = (want.counts + 15) // 16 * 16
+    tiles = sum((((int(c) + 31) // 32) + 4) // 5 for c in padded.tolist())
     assert rows_total[2] == tiles * (N // 512) and rows_total[3] == rows_total[2] * (K // 32)
     sink.zero_()
     ops.grouped_gemm_nn(a, b, got.tile_table)
@@ -175,9 +172,9 @@ def test_clock_hook_counts_workgroups_and_leaves_results_alone(cuda):
 def test_mfma_clock_probe_reports_instructions_and_clocks(cuda):
     import ctypes
 
-    from nestor_amd import _lib
+    from nestor_amd import probes as _lib
 
-    khz = _lib.load().nestor_hip_wall_clock_khz()
+    khz = _lib.wall_clock_khz()
     assert khz > 0
     cus = torch.cuda.get_device_properties(cuda).multi_processor_count
     counters = torch.zeros(4, dtype=torch.int64, device=cuda)
@@ -191,14 +188,17 @@ def test_mfma_clock_probe_reports_instructions_and_clocks(cuda):
         assert cycles >= 500 * 16 * 32 and ticks > 0
         mhz = cycles / ticks * khz / 1000.0
         assert 300 < mhz < 3000
-    with pytest.raises(_lib.NestorHipError):
+    from nestor_amd._lib import NestorHipError
+
+    with pytest.raises(NestorHipError):
         _lib.call("nestor_hip_mfma_clock_probe", 0, 0, ctypes.c_void_p(counters.data_ptr()), None)
 
 
 def test_mfma_mix_probe_counts_and_rejects_bad_arguments(cuda):
     import ctypes
 
-    from nestor_amd import _lib
+    from nestor_amd import probes as _lib
+    from nestor_amd._lib import NestorHipError
 
     cus = torch.cuda.get_device_properties(cuda).multi_processor_count
     region = 1 << 16
@@ -208,7 +208,7 @@ def test_mfma_mix_probe_counts_and_rejects_bad_arguments(cuda):
     plain = None
     for reads, transfers in ((0, 0), (16, 0), (0, 8), (16, 8), (16, 10), (16, 12)):
         _lib.call("nestor_hip_mfma_mix_probe", reads, transfers, 300, ctypes.c_void_p(src.data_ptr()),
-                  region, ctypes.c_void_p(counters.data_ptr()), stream)
+                  src.numel(), region, ctypes.c_void_p(counters.data_ptr()), stream)
         torch.cuda.synchronize()
         cycles, ticks, instructions, _ = counters.tolist()
         assert instructions == cus * 4 * 300 * 32 and ticks > 0
@@ -217,7 +217,11 @@ def test_mfma_mix_probe_counts_and_rejects_bad_arguments(cuda):
             plain = cycles
     # the other instructions cost the wavefront issue cycles: never faster than the bare stream
     assert cycles >= plain
-    for bad in ((8, 8, 300, region), (16, 8, 0, region), (16, 8, 300, 1000), (16, 8, 300, 3 * 32768 + 4096)):
-        with pytest.raises(_lib.NestorHipError):
+    # unsupported mix, no rounds, a region that is not whole 32 KiB steps, a buffer too small
+    # for eight regions: refused on the host, nothing launched
+    for bad in ((8, 8, 300, region, src.numel()), (16, 8, 0, region, src.numel()),
+                (16, 8, 300, 1000, src.numel()), (16, 8, 300, 3 * 32768 + 4096, src.numel()),
+                (16, 8, 300, region, 8 * region - 1)):
+        with pytest.raises(NestorHipError):
             _lib.call("nestor_hip_mfma_mix_probe", bad[0], bad[1], bad[2], ctypes.c_void_p(src.data_ptr()),
-                      bad[3], ctypes.c_void_p(counters.data_ptr()), stream)
+                      bad[4], bad[3], ctypes.c_void_p(counters.data_ptr()), stream)

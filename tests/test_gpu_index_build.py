@@ -26,31 +26,40 @@ def _check(ids2d, num_banks, cuda, capacity=0, dtype=torch.bfloat16):
         w = getattr(want, name)
         assert g.dtype == w.dtype, name
         assert torch.equal(g, w), f"{name} differs (rows={flat.numel()}, E={num_banks}, cap={capacity})"
-    # Tile tables: the 128-row table alone, and the 256-row table together with the
-    # table of remainders, each cover every kept segment exactly once.
+    # Tile tables: each of the three covers every padded row exactly once, no tile crosses
+    # a segment end, and the balanced tables cut a segment of b 32-row blocks into
+    # ceil(b / cap) tiles whose block counts differ by at most one.
     from tests.helpers import tile_tables
 
     tables, _ = tile_tables(got.tile_table, want.rows_pad, num_banks)
     kept = want.counts.clamp(max=capacity) if capacity > 0 else want.counts
     padded = (kept + 15) // 16 * 16
     seg_end_all = int((want.padded_starts + padded)[-1])
-    for parts, limits in (((tables[0],), (128,)), ((tables[1], tables[2]), (256, 128))):
+    for (bank, row0, nrows), cap_blocks in zip(tables, (4, 5, 10)):
         covered = torch.zeros(want.rows_pad, dtype=torch.int32)
-        for (bank, row0, nrows), limit in zip(parts, limits):
-            for b, r0, nr in zip(bank.tolist(), row0.tolist(), nrows.tolist()):
-                assert 0 < nr <= limit
-                covered[r0:r0 + nr] += 1
-                if b >= 0:
-                    assert want.padded_starts[b] <= r0 and r0 + nr <= want.padded_starts[b] + padded[b]
-                else:
-                    assert r0 >= seg_end_all
+        per_bank: dict[int, list[tuple[int, int]]] = {}
+        for b, r0, nr in zip(bank.tolist(), row0.tolist(), nrows.tolist()):
+            assert 0 < nr <= 32 * cap_blocks
+            covered[r0:r0 + nr] += 1
+            if b >= 0:
+                assert want.padded_starts[b] <= r0 and r0 + nr <= want.padded_starts[b] + padded[b]
+                per_bank.setdefault(b, []).append((r0, nr))
+            else:
+                assert r0 >= seg_end_all
         assert torch.equal(covered, torch.ones_like(covered))
-    # a segment contributes floor(len / 256) + (remainder > 128) tiles to the 256-row table
-    # and one remainder tile when 0 < remainder <= 128
-    rem = padded % 256
-    want_256 = int((padded // 256 + (rem > 128).long()).sum())
-    assert int((tables[1][0] >= 0).sum()) == want_256
-    assert len(tables[2][0]) == int(((rem > 0) & (rem <= 128)).sum())
+        for b in range(num_banks):
+            tiles = sorted(per_bank.get(b, []))
+            blocks = (int(padded[b]) + 31) // 32
+            if cap_blocks == 4:
+                assert len(tiles) == (int(padded[b]) + 127) // 128
+                continue
+            assert len(tiles) == (blocks + cap_blocks - 1) // cap_blocks
+            sizes = [(nr + 31) // 32 for _, nr in tiles]
+            assert sum(sizes) == blocks
+            if sizes:
+                assert max(sizes) - min(sizes) <= 1
+                # every tile but a segment's last is made of whole blocks
+                assert all(nr % 32 == 0 for _, nr in tiles[:-1])
     if capacity == 0:
         # The reference kernel's own boundary: maps from a caller-held sort.
         maps = build_dispatch_maps(

@@ -10,8 +10,8 @@ from nestor_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared() -> list[str]:
-    text = open(os.path.join(ROOT, "include", "nestor_hip.h")).read()
+def _declared(header: str = "nestor_hip.h") -> list[str]:
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(nestor_hip_\w+)\s*\(", text)))
 
@@ -24,6 +24,37 @@ def test_header_symbols_exported_and_bound():
     for name in names:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
     assert sorted(_lib.EXPORTED_SYMBOLS) == names, "ctypes table and header disagree"
+
+
+def test_measurement_aids_live_in_their_own_library():
+    """The probes and the instrumented GEMM build are a separate library with its own
+    header; the product library exports none of them."""
+
+    from nestor_amd import build
+
+    probes = _declared("nestor_hip_probes.h")
+    assert "nestor_hip_gemm_clock_sink" in probes and "nestor_hip_mfma_clock_probe" in probes
+    assert build.PROBES_LIB_PATH.exists(), "build the libraries first: python -m nestor_amd.build"
+    plib = ctypes.CDLL(str(build.PROBES_LIB_PATH))
+    for name in probes:
+        assert hasattr(plib, name), f"{name} declared in nestor_hip_probes.h but not exported"
+    # the instrumented GEMM entry points carry the product's names and signatures
+    for name in ("nestor_hip_grouped_gemm_nn", "nestor_hip_grouped_gemm_upgate_swiglu",
+                 "nestor_hip_grouped_gemm_nt", "nestor_hip_grouped_gemm_nt_upgate",
+                 "nestor_hip_grouped_gemm_tn"):
+        assert hasattr(plib, name)
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in probes:
+        assert not hasattr(lib, name), f"{name} leaked into the product library"
+    assert not set(probes) & set(_declared())
+    # the probes that walk a caller's buffer take its size and refuse to leave it
+    null, one = ctypes.c_void_p(0), ctypes.c_void_p(1)
+    i64, i32 = ctypes.c_int64, ctypes.c_int32
+    plib.nestor_hip_dma_stream_probe.argtypes = [ctypes.c_void_p, i64, i64, i64, i32, i32, ctypes.c_void_p]
+    assert plib.nestor_hip_dma_stream_probe(one, 1 << 20, 1024, 8192, 512, 1, null) == -22
+    plib.nestor_hip_mfma_mix_probe.argtypes = [i32, i32, i32, ctypes.c_void_p, i64, i64,
+                                               ctypes.c_void_p, ctypes.c_void_p]
+    assert plib.nestor_hip_mfma_mix_probe(16, 8, 10, one, (8 << 20) - 1, 1 << 20, one, null) == -22
 
 
 def test_version_and_error_strings():
