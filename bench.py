@@ -82,38 +82,40 @@ def _event_ms(fn, iters: int) -> float:
     return start.elapsed_time(end) / iters
 
 
-def routed_private_ids(w, tensors, column_router, pool):
-    """``[T, k_a * k_q]`` private-bank ids and slot weights of the workload's own routers."""
+def routed_slots(w, tensors, column_router, pool):
+    """The workload's own routing: ``(private ids [T, k_a * k_q], private slot weights,
+    public ids [T, k_p], public slot weights)``."""
 
     x3 = tensors.x.view(1, w.tokens, w.d_model)
     valid = torch.ones(1, w.tokens, dtype=torch.bool, device=tensors.x.device)
     with torch.no_grad():
         col = column_router(x3, valid)
-        _pub, privs, stacked, _ = pool._route(x3, valid, col.active_mask)
+        pub, privs, stacked, _ = pool._route(x3, valid, col.active_mask)
         ids, weights, _ = pool._private_slots(privs, col.gates.view(w.tokens, -1), w.tokens,
                                               stacked=stacked)
-    return ids, weights
+        pub_ids, pub_w = pool._public_slots(pub, w.tokens)
+    return ids, weights, pub_ids, pub_w
 
 
-def kernel_breakdown(w, tensors, routed, iters: int = 5) -> dict:
-    """Per-kernel timings of one private-bank call (the larger of the two) on the
-    workload's routed ids, each kernel measured alone with HIP events, against the
-    roofline that bounds it."""
+def bank_call_breakdown(x, grad_out, ids, weights, bank3, iters: int = 5,
+                        gemms_only: bool = False) -> dict:
+    """Per-kernel timings of one bank call (``ids [T, slots]`` into the stacked bank
+    ``bank3 = (w_up, w_gate, w_down)``), each kernel measured alone with HIP events,
+    against the roofline that bounds it.  ``gemms_only``: the grouped GEMMs alone."""
 
-    import ctypes
+    import ctypes  # noqa: F401
 
     from nestor_amd import ops, probes
     from nestor_amd.dispatch import dispatch_plan
 
-    dev = tensors.x.device
-    T, d, h = w.tokens, w.d_model, w.hidden
-    slots = w.k_columns * w.k_private
-    banks = w.columns * w.private
+    dev = x.device
+    T, d = x.shape
+    slots = ids.shape[1]
+    w_up, w_gate, w_down = (t.to(torch.bfloat16) for t in bank3)
+    banks, _, h = w_up.shape
     rows = T * slots
-    g = torch.Generator(device=dev).manual_seed(1)
-    ids = routed[0].reshape(-1).contiguous()
-    weights = routed[1].reshape(-1).to(torch.bfloat16).contiguous()
-    w_up, w_gate, w_down = (t.to(torch.bfloat16) for t in tensors.priv)
+    ids = ids.reshape(-1).contiguous()
+    weights = weights.reshape(-1).to(torch.bfloat16).contiguous()
     out: dict = {}
 
     def report(name, ms, flops=None, bytes_=None):
@@ -147,68 +149,88 @@ def kernel_breakdown(w, tensors, routed, iters: int = 5) -> dict:
             out[name]["shader_mhz"] = round(cycles / ticks * wall_khz / 1000.0)
             out[name]["cycles_per_k_step"] = round(cycles / steps, 1)
 
+    def gemm(name, fn, flops):
+        report(name, _event_ms(fn, iters), flops=flops)
+        shader_clock(name, fn)
+
     plan = dispatch_plan(ids, banks, slots, torch.bfloat16)
     rows_pad = plan.rows_pad
-    ms = _event_ms(lambda: dispatch_plan(ids, banks, slots, torch.bfloat16), iters)
-    report("index_build", ms, bytes_=rows * 8 + rows * 8 + 3 * rows_pad * 8 + rows_pad * 2 + banks * 20)
+    if not gemms_only:
+        ms = _event_ms(lambda: dispatch_plan(ids, banks, slots, torch.bfloat16), iters)
+        report("index_build", ms, bytes_=rows * 8 + rows * 8 + 3 * rows_pad * 8 + rows_pad * 2 + banks * 20)
 
-    x = tensors.x
     x_pad = ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots)
-    ms = _event_ms(lambda: ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots), iters)
-    report("dispatch_fwd", ms, bytes_=T * d * 2 + rows * d * 2 + rows * 8)
+    if not gemms_only:
+        ms = _event_ms(lambda: ops.dispatch_rows_fwd(x, plan.pad_token, plan.pad_valid, plan.row_dest, slots), iters)
+        report("dispatch_fwd", ms, bytes_=T * d * 2 + rows * d * 2 + rows * 8)
 
     up_gate, hidden = ops.upgate_swiglu_fwd(x_pad, w_up, w_gate, plan.tile_table)
-    ms = _event_ms(lambda: ops.upgate_swiglu_fwd(x_pad, w_up, w_gate, plan.tile_table), iters)
-    report("gemm_upgate_swiglu", ms, flops=2.0 * rows * d * 2 * h)
+    gemm("gemm_upgate_swiglu", lambda: ops.upgate_swiglu_fwd(x_pad, w_up, w_gate, plan.tile_table),
+         2.0 * rows * d * 2 * h)
     out["gemm_upgate_swiglu"]["flops_per_launch"] = 2.0 * rows * d * 2 * h
-    out["gemm_upgate_swiglu"]["kernel"] = UPGATE_KERNEL_NAME
-    shader_clock("gemm_upgate_swiglu", lambda: ops.upgate_swiglu_fwd(x_pad, w_up, w_gate, plan.tile_table))
 
     y_pad = ops.grouped_gemm_nn(hidden, w_down, plan.tile_table)
-    ms = _event_ms(lambda: ops.grouped_gemm_nn(hidden, w_down, plan.tile_table), iters)
-    report("gemm_down", ms, flops=2.0 * rows * h * d)
-    shader_clock("gemm_down", lambda: ops.grouped_gemm_nn(hidden, w_down, plan.tile_table))
+    gemm("gemm_down", lambda: ops.grouped_gemm_nn(hidden, w_down, plan.tile_table), 2.0 * rows * h * d)
 
-    o = ops.combine_rows_fwd(y_pad, plan.row_dest, weights, slots, torch.bfloat16, True)
-    ms = _event_ms(lambda: ops.combine_rows_fwd(y_pad, plan.row_dest, weights, slots, torch.bfloat16, True), iters)
-    report("combine_fwd", ms, bytes_=rows * d * 2 + rows * (8 + 2) + (rows // slots) * d * 2)
+    if not gemms_only:
+        o = ops.combine_rows_fwd(y_pad, plan.row_dest, weights, slots, torch.bfloat16, True)
+        ms = _event_ms(lambda: ops.combine_rows_fwd(y_pad, plan.row_dest, weights, slots, torch.bfloat16, True), iters)
+        report("combine_fwd", ms, bytes_=rows * d * 2 + rows * (8 + 2) + (rows // slots) * d * 2)
+        del o
+        ms = _event_ms(lambda: ops.combine_rows_bwd(grad_out, y_pad, plan.pad_src_row, plan.pad_valid, weights, slots, True, plan.row_dest), iters)
+        report("combine_bwd", ms, bytes_=(rows // slots) * d * 2 + rows * d * 2 + rows * d * 2 + rows * 4)
+    gy, _ = ops.combine_rows_bwd(grad_out, y_pad, plan.pad_src_row, plan.pad_valid, weights, slots, True, plan.row_dest)
 
-    go = tensors.grad_out
-    ms = _event_ms(lambda: ops.combine_rows_bwd(go, y_pad, plan.pad_src_row, plan.pad_valid, weights, slots, True, plan.row_dest), iters)
-    report("combine_bwd", ms, bytes_=(rows // slots) * d * 2 + rows * d * 2 + rows * d * 2 + rows * 4)
-    gy, _ = ops.combine_rows_bwd(go, y_pad, plan.pad_src_row, plan.pad_valid, weights, slots, True, plan.row_dest)
-
-    ms = _event_ms(lambda: ops.grouped_gemm_nt(gy, w_down, plan.tile_table), iters)
-    report("gemm_dgrad_down", ms, flops=2.0 * rows * h * d)
-    shader_clock("gemm_dgrad_down", lambda: ops.grouped_gemm_nt(gy, w_down, plan.tile_table))
+    gemm("gemm_dgrad_down", lambda: ops.grouped_gemm_nt(gy, w_down, plan.tile_table), 2.0 * rows * h * d)
     gh = ops.grouped_gemm_nt(gy, w_down, plan.tile_table)
 
-    ms = _event_ms(lambda: ops.grouped_gemm_tn(hidden, gy, plan.offs, plan.padded_starts, plan.counts), iters)
-    report("gemm_wgrad_down", ms, flops=2.0 * rows * h * d)
-    shader_clock("gemm_wgrad_down", lambda: ops.grouped_gemm_tn(hidden, gy, plan.offs, plan.padded_starts, plan.counts))
+    gemm("gemm_wgrad_down", lambda: ops.grouped_gemm_tn(hidden, gy, plan.offs, plan.padded_starts, plan.counts),
+         2.0 * rows * h * d)
 
-    ms = _event_ms(lambda: ops.swiglu_bwd(gh, up_gate, h), iters)
-    report("swiglu_bwd", ms, bytes_=rows * h * 2 * (1 + 2 + 2))
+    if not gemms_only:
+        ms = _event_ms(lambda: ops.swiglu_bwd(gh, up_gate, h), iters)
+        report("swiglu_bwd", ms, bytes_=rows * h * 2 * (1 + 2 + 2))
     gug = ops.swiglu_bwd(gh, up_gate, h)
 
-    ms = _event_ms(lambda: ops.grouped_gemm_nt_upgate(gug, w_up, w_gate, plan.tile_table), iters)
-    report("gemm_dgrad_upgate", ms, flops=2.0 * rows * d * 2 * h)
-    shader_clock("gemm_dgrad_upgate", lambda: ops.grouped_gemm_nt_upgate(gug, w_up, w_gate, plan.tile_table))
+    gemm("gemm_dgrad_upgate", lambda: ops.grouped_gemm_nt_upgate(gug, w_up, w_gate, plan.tile_table),
+         2.0 * rows * d * 2 * h)
     gx_pad = ops.grouped_gemm_nt_upgate(gug, w_up, w_gate, plan.tile_table)
 
-    ms = _event_ms(lambda: ops.grouped_gemm_tn(x_pad, gug[:, :h], plan.offs, plan.padded_starts, plan.counts), iters)
-    report("gemm_wgrad_up(one of 2)", ms, flops=2.0 * rows * d * h)
-    shader_clock("gemm_wgrad_up(one of 2)", lambda: ops.grouped_gemm_tn(x_pad, gug[:, :h], plan.offs, plan.padded_starts, plan.counts))
+    gemm("gemm_wgrad_up(one of 2)",
+         lambda: ops.grouped_gemm_tn(x_pad, gug[:, :h], plan.offs, plan.padded_starts, plan.counts),
+         2.0 * rows * d * h)
+    if gemms_only:
+        return out
 
     ms = _event_ms(lambda: ops.dispatch_rows_bwd(gx_pad, plan.row_dest, T, slots, torch.bfloat16), iters)
     report("dispatch_bwd", ms, bytes_=rows * d * 2 + T * d * 2)
-    del o
 
     # biased banks: the bias gradient as a segmented column sum over the padded rows
     ms = _event_ms(lambda: ops.segment_colsum(gh, None, plan.padded_starts, plan.counts), iters)
     report("bias_grad_colsum", ms, bytes_=rows * h * 2)
+    out["_scratch"] = gx_pad  # reused by the caller for the pool epilogue rows
+    return out
+
+
+def kernel_breakdown(w, tensors, routed, iters: int = 5) -> dict:
+    """Per-kernel timings of one private-bank call (the larger of the two) on the
+    workload's routed ids, plus the pool's epilogue kernels."""
+
+    from nestor_amd import ops
+
+    dev = tensors.x.device
+    T, d = w.tokens, w.d_model
+    x, go = tensors.x, tensors.grad_out
+    out = bank_call_breakdown(x, go, routed[0], routed[1], tensors.priv, iters)
+    out["gemm_upgate_swiglu"]["kernel"] = UPGATE_KERNEL_NAME
+    gx_pad = out.pop("_scratch")
+
+    def report(name, ms, bytes_):
+        gbs = bytes_ / ms / 1e6
+        out[name] = {"ms": round(ms, 4), "gbs": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
 
     # pool epilogues: the summed layout's path mix and the column layout's scatter
+    g = torch.Generator(device=dev).manual_seed(1)
     alpha = torch.softmax(torch.randn(T, 2, generator=g, device=dev), -1).to(torch.bfloat16)
     pub, priv = x, gx_pad[:T]
     ms = _event_ms(lambda: ops.path_mix_fwd(pub, priv, alpha), iters)
@@ -223,6 +245,70 @@ def kernel_breakdown(w, tensors, routed, iters: int = 5) -> dict:
     g_cols = ops.path_scale_fwd(per_slot, alpha, 1, columns, w.columns)
     ms = _event_ms(lambda: ops.path_scale_bwd(g_cols, per_slot, alpha, 1, columns), iters)
     report("column_scatter_bwd", ms, bytes_=3 * T * k_a * d * 2)
+    return out
+
+
+def timed_steps(w, column_router, pool, x, grad_out, steps: int, warmup: int, autocast: bool) -> float:
+    """ms per step of the whole path (forward + backward), host clock around ``steps``
+    steps bracketed by device synchronisations."""
+
+    from nestor_amd.workloads import expert_mlp_step
+
+    params = list(column_router.parameters()) + list(pool.parameters())
+
+    def step():
+        for p in params:
+            p.grad = None
+        x.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            expert_mlp_step(w, column_router, pool, x, grad_out)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    for p in params:
+        p.grad = None
+    x.grad = None
+    return ms
+
+
+def extra_shapes(dev, seed: int) -> dict:
+    """The path at the reference's production widths (registered ``nestor_*`` arms: d that
+    is no power of two, private widths of 160-424, 6-16 slots per token, 120 private
+    experts): ms per step and the grouped GEMMs of both bank calls against the MFMA peak.
+    Not the headline: BASELINE's configuration is ``mlp_1b``."""
+
+    from nestor_amd.workloads import WORKLOADS, build_pool, make_tensors
+
+    out = {}
+    for name in ("nestor_1b_block0", "nestor_1b_block6", "nestor_200m_block0"):
+        w = WORKLOADS[name]
+        t = make_tensors(w, seed, dev)
+        column_router, pool = build_pool(w, t)
+        x = t.x.clone().requires_grad_(True)
+        ms = timed_steps(w, column_router, pool, x, t.grad_out, 5, 2, False)
+        flops = w.gemm_flops()
+        routed = routed_slots(w, t, column_router, pool)
+        entry = {
+            "shape": f"T={w.tokens} d={w.d_model} private {w.columns}x{w.private} h={w.hidden} "
+                     f"top-{w.k_columns} columns x top-{w.k_private} = {w.k_columns * w.k_private} slots; "
+                     f"public {w.public} h={w.h_public} top-{w.k_public}",
+            "ms_per_step": round(ms, 3),
+            "tokens_per_s": round(w.tokens / ms * 1e3, 1),
+            "expert_gemm_tflops": round(flops / ms / 1e9, 1),
+            "expert_gemm_frac_mfma_peak": round(flops / ms / 1e9 / BF16_MFMA_PEAK_TFLOPS, 4),
+        }
+        for call, ids, wts, bank3 in (("private", routed[0], routed[1], t.priv), ("public", routed[2], routed[3], t.pub)):
+            rows = bank_call_breakdown(t.x, t.grad_out, ids, wts, bank3, 5, gemms_only=True)
+            entry[f"{call}_gemms"] = {k: {"ms": v["ms"], "frac_mfma_peak": v["frac_mfma_peak"]} for k, v in rows.items()}
+        out[name] = entry
+        del t, pool, column_router, x
+        torch.cuda.empty_cache()
     return out
 
 
@@ -489,6 +575,8 @@ def main() -> None:
                          "keeping the persistent bf16 copy")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the fp32-owner step and the production-shape figures")
     ap.add_argument("--no-fp8", action="store_true",
                     help="skip the e4m3 inference-regime figures (64 / 256 / 1024 tokens)")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -506,7 +594,7 @@ def main() -> None:
         sys.exit("bench.py needs a GPU (the HIP kernels have no CPU fallback)")
 
     from nestor_amd import _lib
-    from nestor_amd.workloads import WORKLOADS, build_pool, expert_mlp_step, make_tensors
+    from nestor_amd.workloads import WORKLOADS, build_pool, make_tensors
 
     _lib.load()
     _log("library loaded; building workload")
@@ -518,7 +606,7 @@ def main() -> None:
     if fp32_owners and not args.no_shadow:
         pool.enable_bf16_shadow()
     with torch.autocast("cuda", dtype=torch.bfloat16, enabled=fp32_owners):
-        routed = routed_private_ids(w, tensors, column_router, pool)
+        routed = routed_slots(w, tensors, column_router, pool)
     if args.traffic_probe:
         traffic_probe(w, tensors, routed)
         return
@@ -527,39 +615,15 @@ def main() -> None:
                           "unit": "GB/s of weight bytes streamed",
                           "tokens": fp8_probe(w, tensors, column_router, pool)}))
         return
-    params = list(column_router.parameters()) + list(pool.parameters())
     x = tensors.x.clone().requires_grad_(True)
     grad_out = tensors.grad_out if w.backward else None
-
-    def step():
-        for p in params:
-            p.grad = None
-        x.grad = None
-        if fp32_owners:
-            with torch.autocast("cuda", dtype=torch.bfloat16):
-                expert_mlp_step(w, column_router, pool, x, grad_out)
-        else:
-            expert_mlp_step(w, column_router, pool, x, grad_out)
-
-    _log("workload resident; warm-up")
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    _log("timing")
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    tokens_per_s = w.tokens * args.steps / elapsed
+    _log("workload resident; warm-up and timing")
+    ms_per_step = timed_steps(w, column_router, pool, x, grad_out, args.steps, args.warmup, fp32_owners)
+    tokens_per_s = w.tokens / ms_per_step * 1e3
     flops = w.gemm_flops()
     step_tflops = flops / (ms_per_step * 1e-3) / 1e12
 
     _log(f"{ms_per_step:.3f} ms/step; per-kernel breakdown")
-    for p in params:
-        p.grad = None
-    x.grad = None
     breakdown = {} if args.no_breakdown else kernel_breakdown(w, tensors, routed)
     dom = breakdown.get("gemm_upgate_swiglu")
     roofline = None
@@ -609,7 +673,24 @@ def main() -> None:
                         "further launches (the published peak assumes 2400 MHz)",
     }
     if not args.no_breakdown:
+        # the public bank call's GEMMs (slots = 1, 16 banks of ~2048 rows) beside the private ones
+        result["kernels_public"] = bank_call_breakdown(
+            tensors.x, tensors.grad_out, routed[2], routed[3], tensors.pub, 5, gemms_only=True)
         result["mfma_clock_probe"] = mfma_clock_probe(dev)
+    if not args.no_extra and w.name == "mlp_1b" and not fp32_owners:
+        # the production dtype flow: fp32 owners under bf16 autocast, the GEMMs reading a
+        # persistent bf16 copy and the weight gradient written as fp32 into the owners' .grad
+        _log("fp32-owner flow")
+        t32 = make_tensors(w, args.seed, dev, torch.float32)
+        router32, pool32 = build_pool(w, t32)
+        pool32.enable_bf16_shadow()
+        x32 = t32.x.clone().requires_grad_(True)
+        result["fp32_owner_ms_per_step"] = round(
+            timed_steps(w, router32, pool32, x32, t32.grad_out, 5, 2, True), 3)
+        del t32, router32, pool32, x32
+        torch.cuda.empty_cache()
+        _log("production shapes")
+        result["extra_shapes"] = extra_shapes(dev, args.seed)
     if not args.no_fp8 and w.name == "mlp_1b" and not fp32_owners:
         _log("e4m3 inference regime")
         del x

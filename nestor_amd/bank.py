@@ -160,12 +160,29 @@ class StackedExpertBank(nn.Module):
         gradient, and the copy is rebuilt only when an owner has changed (an
         optimizer step bumps the tensor's version counter; ``refresh_shadow()``
         forces it) -- the arrangement of nestor/scaling/bf16_master.py:1-40 seen
-        from the other side: fp32 masters stay the parameters, bf16 is the cache."""
+        from the other side: fp32 masters stay the parameters, bf16 is the cache.
+
+        What the version counter does not see is a write through ``.data``
+        (``p.data.copy_(...)`` leaves ``p._version`` alone), and the reference writes
+        owners exactly that way: the EMA swap around evaluation
+        (nestor/train/trainer.py:974-999) and the master restore of a resumed Muon
+        state (nestor/scaling/muon.py:582).  Therefore: in evaluation mode the copy is
+        rebuilt on EVERY call (evaluation is where the EMA weights are swapped in and
+        out with no mode change in between, trainer.py:557-563; one cast per bank call
+        is what the path without a shadow pays anyway); every ``train()`` / ``eval()``
+        transition and every ``load_state_dict`` drops the copy; and code that writes
+        an owner through ``.data`` while the module stays in training mode (the Muon
+        resume, when a forward has already run) must call ``refresh_shadow()``."""
 
         self.__dict__["_shadow_enabled"] = bool(enabled)
         if not enabled:
             self.__dict__.pop("_shadow", None)
         return self
+
+    def invalidate_shadow(self) -> None:
+        """Forget the bf16 copies; the next bank call rebuilds them from the owners."""
+
+        self.__dict__.pop("_shadow", None)
 
     def refresh_shadow(self) -> None:
         """Rebuild the bf16 copies from the owners now."""
@@ -175,6 +192,15 @@ class StackedExpertBank(nn.Module):
             copies = tuple(None if o is None else o.detach().to(torch.bfloat16) for o in owners)
         key = tuple(None if o is None else (o.data_ptr(), o._version) for o in owners)
         self.__dict__["_shadow"] = (key, copies)
+
+    def train(self, mode: bool = True):
+        if bool(mode) != self.training:
+            self.invalidate_shadow()
+        return super().train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self.invalidate_shadow()
+        return super()._load_from_state_dict(*args, **kwargs)
 
     def shadowed(self, dtype: torch.dtype):
         """``((w_up, w_gate, w_down) bf16 copies, (owner_up, owner_gate, owner_down))`` when
@@ -188,7 +214,7 @@ class StackedExpertBank(nn.Module):
         owners = (self.w_up, self.w_gate, self.w_down)
         key = tuple(None if o is None else (o.data_ptr(), o._version) for o in owners)
         cached = self.__dict__.get("_shadow")
-        if cached is None or cached[0] != key:
+        if cached is None or cached[0] != key or not self.training:
             self.refresh_shadow()
             cached = self.__dict__["_shadow"]
         return cached[1], owners

@@ -414,13 +414,9 @@ int launch_fp8_stream(GemmParams p, void* stream) {
   p.n_tiles = static_cast<int>(p.N / (kUpGate ? C::BN / 2 : C::BN));
   int64_t blocks = p.max_tiles * p.n_tiles;
   if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
-  static bool configured = false;
-  if (!configured) {
-    (void)hipFuncSetAttribute(
-        reinterpret_cast<const void*>(fp8w_stream_kernel<kMi, kStages, kUpGate, kW, kBN>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(C::LDS_BYTES));
-    configured = true;
-  }
+  static const bool configured = allow_dynamic_lds(
+      reinterpret_cast<const void*>(fp8w_stream_kernel<kMi, kStages, kUpGate, kW, kBN>), C::LDS_BYTES);
+  (void)configured;
   // Persistent workgroups, as many per CU as the ring's LDS allows; fewer when the
   // launch cannot have that many items.
   const int cus = cu_count();

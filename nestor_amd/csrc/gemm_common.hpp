@@ -317,17 +317,24 @@ inline bool dims_ok(int64_t rows_pad, int64_t K, int64_t N, int32_t num_banks, i
          max_tiles == table_cap(kTiles128, rows_pad, num_banks);
 }
 
-// Compute units of the current device (0 if the query fails).
+// Compute units of the current device (0 if the query fails).  Initialised once, by
+// whichever thread comes first (function-local statics are thread-safe).
 inline int cu_count() {
-  static int cus = -1;
-  if (cus < 0) {
+  static const int cus = [] {
     int dev = 0;
     hipDeviceProp_t prop;
-    cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-              ? prop.multiProcessorCount
-              : 0;
-  }
+    return (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+               ? prop.multiProcessorCount
+               : 0;
+  }();
   return cus;
+}
+
+// Raises a kernel's dynamic LDS limit; meant as the initialiser of a function-local
+// static of each launcher, so that it runs once per kernel and is safe to race into.
+inline bool allow_dynamic_lds(const void* kernel, size_t bytes) {
+  (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+  return true;
 }
 
 // The register-staged e4m3-weight kernel (128-row tiles, weights widened on the way into

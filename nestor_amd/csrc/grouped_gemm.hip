@@ -550,14 +550,6 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       tile = (group * 8 + xcd) * p.tile_group + within % p.tile_group;
       nt = within / p.tile_group;
     }
-  } else if (p.tile_order == 2) {
-    // every XCD keeps n_tiles / 8 ADJACENT column tiles of every row tile (the launcher
-    // checks that n_tiles is a multiple of 8): with column tiles dealt x, x + 8, ... the
-    // XCDs with the even ones ran 6 % longer than the others and the launch waited for them
-    const int per = p.n_tiles >> 3;
-    const int seq = blockIdx.x >> 3;
-    tile = seq / per;
-    nt = (blockIdx.x & 7) * per + seq % per;
   } else {
     tile = blockIdx.x / p.n_tiles;
     nt = blockIdx.x % p.n_tiles;
@@ -1369,13 +1361,9 @@ int launch_rows(GemmParams p, void* stream) {
   p.n_tiles = static_cast<int>(ceil_div(p.N, out_cols));
   const int64_t blocks = p.max_tiles * p.n_tiles;
   if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
-  static bool configured = false;
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_kernel<C, kMode>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(C::LDS_BYTES));
-    configured = true;
-  }
+  static const bool configured = allow_dynamic_lds(
+      reinterpret_cast<const void*>(grouped_gemm_kernel<C, kMode>), C::LDS_BYTES);
+  (void)configured;
   hipLaunchKernelGGL((grouped_gemm_kernel<C, kMode>), dim3(static_cast<unsigned>(blocks)),
                      dim3(kThreads), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
   return launch_status();
@@ -1412,18 +1400,13 @@ int launch_rows_dma(GemmParams p, int table_kind, int64_t rows_pad, int32_t num_
   p.tile_group = forced_group >= 0 ? forced_group : (kMode == kNN ? 8 : kMode == kNTUpGate ? 4 : 0);
   static const int forced_order = config_choice("NESTOR_HIP_TILE_ORDER", -1);
   p.tile_order = forced_order >= 0 ? forced_order : (kMode == kNN ? 1 : 0);
-  if (p.tile_order == 2 && (p.tile_group > 0 || p.n_tiles % 8 != 0)) p.tile_order = 0;
   // whole groups of row tiles per XCD (see the kernel's tile mapping)
   const int64_t gran = p.tile_group > 0 ? 8 * p.tile_group : 1;
   const int64_t blocks = ceil_div(p.max_tiles, gran) * gran * p.n_tiles;
   if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
-  static bool configured = false;
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_dma_kernel<C, kMode>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(C::LDS_BYTES));
-    configured = true;
-  }
+  static const bool configured = allow_dynamic_lds(
+      reinterpret_cast<const void*>(grouped_gemm_dma_kernel<C, kMode>), C::LDS_BYTES);
+  (void)configured;
   hipLaunchKernelGGL((grouped_gemm_dma_kernel<C, kMode>), dim3(static_cast<unsigned>(blocks)),
                      dim3(C::THREADS), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
   return launch_status();
@@ -1471,13 +1454,9 @@ int dispatch_rows_gemm(const GemmParams& p, int64_t rows_pad, int32_t num_banks,
 
 template <typename C>
 int launch_wgrad(const GemmParams& p, int32_t num_banks, void* stream) {
-  static bool configured = false;
-  if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(grouped_gemm_kernel<C, kTN>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(C::LDS_BYTES));
-    configured = true;
-  }
+  static const bool configured = allow_dynamic_lds(
+      reinterpret_cast<const void*>(grouped_gemm_kernel<C, kTN>), C::LDS_BYTES);
+  (void)configured;
   const int64_t my = ceil_div(p.M, C::BM);
   if (my > 65535) return NESTOR_HIP_ERANGE;
   hipLaunchKernelGGL((grouped_gemm_kernel<C, kTN>),
@@ -1625,20 +1604,13 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
   const bool spans_fit = rows_pad * lda * 2 < (int64_t{1} << 32) && rows_pad * ldg * 2 < (int64_t{1} << 32);
   if (cfg == 5 && M >= 256 && N >= 256 && rows_pad <= INT32_MAX && spans_fit) {
     using C = WgradPers;
-    static int num_cus = 0;
-    if (num_cus == 0) {
-      int dev = 0;
-      hipDeviceProp_t prop;
-      if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-        return NESTOR_HIP_ELAUNCH;
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(WgradLayout<C>::LDS_BYTES));
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(WgradLayout<C>::LDS_BYTES));
-      num_cus = prop.multiProcessorCount / 8 * 8;
-    }
+    static const bool configured =
+        allow_dynamic_lds(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, false>),
+                          WgradLayout<C>::LDS_BYTES) &&
+        allow_dynamic_lds(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, true>),
+                          WgradLayout<C>::LDS_BYTES);
+    (void)configured;
+    const int num_cus = cu_count() / 8 * 8;
     const int64_t items = ceil_div(M, C::BM) * ceil_div(N, C::BN) * num_banks;
     if (num_cus >= 8 && items / num_cus + 2 <= WgradLayout<C>::kMaxItems) {
 #if NESTOR_GEMM_CLOCK_HOOK

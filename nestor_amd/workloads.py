@@ -34,6 +34,11 @@ class Workload:
     k_private: int = 1
     k_public: int = 1
     backward: bool = True
+    hidden_public: int = 0   # 0: the public experts are as wide as the private ones
+
+    @property
+    def h_public(self) -> int:
+        return self.hidden_public or self.hidden
 
     @property
     def experts(self) -> int:
@@ -47,7 +52,8 @@ class Workload:
         """``2 * rows * K * N`` per GEMM over real rows: forward ``18 T d h`` at three
         assignments per token, backward twice that."""
 
-        fwd = 6.0 * self.assignments * self.tokens * self.d_model * self.hidden
+        per_token = (self.k_public * self.h_public + self.k_columns * self.k_private * self.hidden)
+        fwd = 6.0 * self.tokens * self.d_model * per_token
         bwd = self.backward if backward is None else backward
         return fwd * (3.0 if bwd else 1.0)
 
@@ -56,6 +62,17 @@ WORKLOADS = {
     "tiny_100m": Workload("tiny_100m", 4096, 512, 1024, 4, 8, 2, 0.02, backward=False),
     "mlp_200m": Workload("mlp_200m", 16384, 1024, 2048, 8, 16, 4, 0.02),
     "mlp_1b": Workload("mlp_1b", 32768, 2048, 4096, 16, 32, 4, 0.014),
+    # The reference's registered arms at their real widths (experiments/pretrain.py:145-150,
+    # 174-193; width contract expert_pool_dispatch.py:38-105): 8 columns, top-k columns and
+    # private top-k per block, 8 public experts top-2 of width d, 4 x 4096 tokens per
+    # micro-batch.  One entry per block shape that differs in kind: the widest private
+    # experts with the fewest slots per token, and the narrowest with the most.
+    "nestor_1b_block0": Workload("nestor_1b_block0", 16384, 1280, 424, 8, 8, 15, 0.02,
+                                 k_columns=3, k_private=2, k_public=2, hidden_public=1280),
+    "nestor_1b_block6": Workload("nestor_1b_block6", 16384, 1280, 160, 8, 8, 15, 0.02,
+                                 k_columns=8, k_private=2, k_public=2, hidden_public=1280),
+    "nestor_200m_block0": Workload("nestor_200m_block0", 16384, 640, 216, 8, 8, 8, 0.02,
+                                   k_columns=3, k_private=2, k_public=2, hidden_public=640),
 }
 
 
@@ -84,11 +101,11 @@ def make_tensors(w: Workload, seed: int, device: torch.device | str,
             return out
         return (torch.randn(shape, generator=g, device=device) * std).to(dtype)
 
-    def bank(n: int) -> tuple[Tensor, Tensor, Tensor]:
+    def bank(n: int, hidden: int) -> tuple[Tensor, Tensor, Tensor]:
         return (
-            randn(n, w.d_model, w.hidden, std=w.weight_std, dtype=weight_dtype),
-            randn(n, w.d_model, w.hidden, std=w.weight_std, dtype=weight_dtype),
-            randn(n, w.hidden, w.d_model, std=w.weight_std, dtype=weight_dtype),
+            randn(n, w.d_model, hidden, std=w.weight_std, dtype=weight_dtype),
+            randn(n, w.d_model, hidden, std=w.weight_std, dtype=weight_dtype),
+            randn(n, hidden, w.d_model, std=w.weight_std, dtype=weight_dtype),
         )
 
     x = randn(w.tokens, w.d_model, dtype=torch.bfloat16)
@@ -97,7 +114,7 @@ def make_tensors(w: Workload, seed: int, device: torch.device | str,
     w_public = randn(w.public, w.d_model, std=w.router_std)
     w_private = randn(w.columns, w.private, w.d_model, std=w.router_std)
     return WorkloadTensors(x, grad_out, w_columns, w_public, w_private,
-                           bank(w.public), bank(w.columns * w.private))
+                           bank(w.public, w.h_public), bank(w.columns * w.private, w.hidden))
 
 
 def build_pool(w: Workload, t: WorkloadTensors):

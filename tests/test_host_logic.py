@@ -187,3 +187,44 @@ def test_training_noise_is_refused_not_ignored():
     with pytest.raises(NotImplementedError):
         na.route_private_batched(list(pool.private_routers), args[0], args[1], args[3], training=True,
                                  noise=torch.zeros(1))
+
+
+def test_bf16_shadow_follows_data_writes():
+    """The persistent bf16 copy of fp32 owners must not go stale when an owner is written
+    through ``.data`` -- how the reference swaps EMA weights in and out around evaluation
+    (nestor/train/trainer.py:974-999) and restores Muon masters on resume
+    (nestor/scaling/muon.py:582) -- which leaves the tensor's version counter alone."""
+
+    from nestor_amd.bank import StackedExpertBank
+
+    g = torch.Generator().manual_seed(0)
+    w3 = [torch.randn(3, a, b, generator=g) for a, b in ((8, 16), (8, 16), (16, 8))]
+    bank = StackedExpertBank.from_tensors(*[t.clone() for t in w3]).enable_bf16_shadow()
+
+    def copies():
+        return bank.shadowed(torch.bfloat16)[0]
+
+    first = copies()
+    assert all(torch.equal(c, w.bfloat16()) for c, w in zip(first, w3))
+    assert copies()[0] is first[0]                       # training mode, untouched owners: cached
+    with torch.no_grad():
+        bank.w_up.mul_(2.0)                              # optimizer-style update: version bump
+    assert torch.equal(copies()[0], (w3[0] * 2).bfloat16())
+    # the EMA swap: eval, .data write, eval again with no mode change, .data write back, train
+    version = bank.w_down._version
+    bank.eval()
+    live = copies()[2].clone()
+    bank.w_down.data.copy_(w3[2] * 3)
+    assert bank.w_down._version == version               # invisible to the version counter ...
+    assert torch.equal(copies()[2], (w3[2] * 3).bfloat16())   # ... and still picked up
+    bank.w_down.data.copy_(w3[2])
+    bank.train()
+    assert torch.equal(copies()[2], live)
+    # a .data write in training mode is the documented case for refresh_shadow()
+    bank.w_gate.data.copy_(w3[1] * 5)
+    bank.refresh_shadow()
+    assert torch.equal(copies()[1], (w3[1] * 5).bfloat16())
+    # loading a state dict drops the copy
+    state = {k: v.clone() * 0.5 for k, v in bank.state_dict().items()}
+    bank.load_state_dict(state)
+    assert torch.equal(copies()[0], state["w_up"].bfloat16())

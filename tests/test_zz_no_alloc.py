@@ -88,3 +88,52 @@ def test_static_scratch_limit_is_refused(cuda):
         ctypes.c_void_p(ids.data_ptr()), rows, num_banks, 1, rows_pad, 0, _lib.BF16, *ptr,
         max_tiles, ctypes.c_void_p(torch.cuda.current_stream(cuda).cuda_stream))
     assert status == -34
+
+
+def test_static_entry_allocates_nothing(cuda):
+    """The entry point is for callers that cannot allocate.  Two observations: the device's
+    free memory is the same before and after a call (``hipMemGetInfo``), and the call can be
+    recorded into a HIP graph -- capture refuses allocations -- whose replays (with eager
+    work and synchronisations in between) give the workspace entry point's results."""
+
+    g = torch.Generator().manual_seed(9)
+    tokens, slots, num_banks = 4096, 2, 32
+    ids = torch.randint(0, num_banks, (tokens * slots,), generator=g).to(cuda)
+    want = _run("nestor_hip_index_build", ids, num_banks, slots, 0)
+    _run("nestor_hip_index_build_static", ids, num_banks, slots, 0)   # set-up happens here, once
+    outs, rows_pad, max_tiles = _outputs(tokens * slots, num_banks, cuda)
+    ptr = [ctypes.c_void_p(t.data_ptr()) for t in outs]
+    lib = _lib.load()
+
+    def call(stream):
+        status = lib.nestor_hip_index_build_static(
+            ctypes.c_void_p(ids.data_ptr()), tokens * slots, num_banks, slots, rows_pad, 0, _lib.BF16,
+            *ptr, max_tiles, ctypes.c_void_p(stream.cuda_stream))
+        assert status == 0
+
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(cuda)
+    call(torch.cuda.current_stream(cuda))
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(cuda)
+    assert free_after == free_before
+
+    from tests.helpers import tile_tables
+
+    def check():
+        torch.cuda.synchronize()
+        got = list(outs)
+        got[11] = tile_tables(got[11], rows_pad, num_banks)[1]
+        for name, a, b in zip(_NAMES, got, want):
+            assert torch.equal(a, b), name
+
+    check()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream(cuda))
+    for _ in range(3):
+        for t in outs:
+            t.fill_(-3)                       # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        check()
