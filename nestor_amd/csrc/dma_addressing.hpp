@@ -60,6 +60,25 @@ NESTOR_HD uint32_t b_major_lane_offset(int ci, int64_t n0, int64_t N, int64_t ld
   return static_cast<uint32_t>((static_cast<int64_t>(k) * ldb + (n - n0)) * 2);
 }
 
+// ---- the last K step of a contraction that is not a multiple of BK -------------
+// k_rem = K % BK valid contraction indices (a multiple of 8, > 0).  Every lane still
+// fetches 16 bytes that lie inside the operand (and hold finite values): a piece
+// behind k_rem is replaced by one in front of it, and what the replaced pieces feed is
+// cancelled by zeroing the A fragments of those contraction indices in registers.
+// Each function returns how many bytes to SUBTRACT from the regular lane offset.
+template <int BK>
+NESTOR_HD uint32_t kc_partial_adjust(int ci, int k_rem) {
+  int row, c;
+  kc_piece_of<BK>(ci, row, c);
+  return c * 8 < k_rem ? 0u : static_cast<uint32_t>(c * 16);  // piece 0 of the same row
+}
+template <int BK, int BW>
+NESTOR_HD uint32_t b_major_partial_adjust(int ci, int k_rem, int64_t ldb) {
+  constexpr int kPerSub = BK * BW / 8;
+  const int k = (ci % kPerSub) / (BW / 8);
+  return k < k_rem ? 0u : static_cast<uint32_t>(static_cast<int64_t>(k - (k_rem - 1)) * ldb * 2);  // row k_rem - 1
+}
+
 // ---- persistent weight gradient ----------------------------------------------
 // Both operands are [segment row, column] with 256-column tiles: one transfer covers
 // two contraction rows x 32 pieces.

@@ -502,7 +502,13 @@ __device__ __forceinline__ void mfma_vgpr(f32x16& c, bf16x8 a, bf16x8 b) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
 }
 
-template <typename C, int kMode>
+// kRagK: the contraction length is not a multiple of BK (any multiple of 8 goes).  The
+// last K step of each phase then fetches, in place of the pieces behind the
+// contraction's end, pieces in front of it (finite values from inside the operand) and
+// multiplies them with A fragments zeroed in registers; the per-transfer offset
+// correction costs two vector instructions per transfer, which is why contractions
+// that are multiples of BK keep the variant without it.
+template <typename C, int kMode, bool kRagK>
 __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(GemmParams p) {
   static_assert(kMode != kTN && kMode != kNNFp8W, "row-tiled bf16 modes");
   constexpr int kThreads = C::THREADS, kWaves = C::WAVES;
@@ -582,8 +588,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     return;
   }
 
-  const int kt_per_phase = static_cast<int>(p.K / BK);
+  const int kt_per_phase = static_cast<int>((p.K + BK - 1) / BK);
   const int num_kt = kMode == kNTUpGate ? 2 * kt_per_phase : kt_per_phase;
+  const int k_rem = static_cast<int>(p.K % BK);  // kRagK: valid contraction indices of a phase's last step
 #if NESTOR_GEMM_CLOCK_HOOK
   unsigned long long clk_c0 = 0, clk_w0 = 0;
   if (p.clock_sink != nullptr) {
@@ -615,6 +622,19 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     if constexpr (kBContig) offb[i] = dma::b_contig_lane_offset<BK>(ci, n0, p.N, p.ldb);
     else offb[i] = dma::b_major_lane_offset<BK, BW>(ci, n0, p.N, p.ldb);
   }
+  // kRagK: what a phase's last K step subtracts from those offsets
+  uint32_t adja[kRagK ? C::A_CHUNKS : 1], adjb[kRagK ? C::B_CHUNKS : 1];
+  if constexpr (kRagK) {
+#pragma unroll
+    for (int i = 0; i < C::A_CHUNKS; ++i)
+      adja[i] = dma::kc_partial_adjust<BK>((wave + kWaves * i) * 64 + lane, k_rem);
+#pragma unroll
+    for (int i = 0; i < C::B_CHUNKS; ++i) {
+      const int ci = (wave + kWaves * i) * 64 + lane;
+      if constexpr (kBContig) adjb[i] = dma::kc_partial_adjust<BK>(ci, k_rem);
+      else adjb[i] = dma::b_major_partial_adjust<BK, BW>(ci, k_rem, p.ldb);
+    }
+  }
   const uint16_t* a_origin = p.a + static_cast<int64_t>(row0) * p.lda;
   const int64_t b_origin = bank * p.bank_stride + (kBContig ? n0 * p.ldb : n0);
 
@@ -637,8 +657,21 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     constexpr int q = decltype(q_tag)::value;
     kt = kt < num_kt ? kt : num_kt - 1;
     const uint32_t stage_lds = wave_lds + stage * (kStageElems * 2);
+    // all ones in a phase's last (partial) K step, else zero: wavefront-uniform
+    uint32_t part = 0;
+    uint32_t a_col_bytes = static_cast<uint32_t>(kt) * a_step;
+    if constexpr (kRagK) {
+      const int phase = (kMode == kNTUpGate && kt >= kt_per_phase) ? 1 : 0;
+      const int in_phase = kt - phase * kt_per_phase;
+      part = in_phase == kt_per_phase - 1 ? 0xffffffffu : 0u;
+      // the second phase's columns start at K, which is not a whole number of K steps here
+      a_col_bytes = static_cast<uint32_t>(phase) * static_cast<uint32_t>(p.K * 2) +
+                    static_cast<uint32_t>(in_phase) * a_step;
+    }
     if constexpr (q < kA) {
-      dma16s<q * kWaves * 1024>(a_bytes + static_cast<uint32_t>(kt) * a_step, offa[q], stage_lds);
+      uint32_t off = offa[q];
+      if constexpr (kRagK) off -= adja[q] & part;
+      dma16s<q * kWaves * 1024>(a_bytes + a_col_bytes, off, stage_lds);
     } else {
       constexpr int i = q - kA;
       constexpr int kLdsOff = C::A_ELEMS * 2 + i * kWaves * 1024;
@@ -655,7 +688,9 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
         constexpr bool kSecond = kSub == 2 && i * kWaves >= kBlkPerSub;
         base = (kSecond ? b1_bytes : b0_bytes) + static_cast<uint32_t>(kt) * b_step;
       }
-      dma16s<kLdsOff>(base, offb[i], stage_lds);
+      uint32_t off = offb[i];
+      if constexpr (kRagK) off -= adjb[i] & part;
+      dma16s<kLdsOff>(base, off, stage_lds);
     }
   };
 
@@ -710,8 +745,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
   // wavefront's matrix instructions behind them.
   // mi_tag: how many of the wavefront's 32-row blocks hold rows of the tile; the
   // MFMAs and A fragments of the others are skipped.
+  // ckk: the K sub-step (of 16) whose fragments this block multiplies when its K step is a
+  // phase's partial last one, else -1 (kRagK only).
   auto mfma_block = [&](auto mi_tag, int par, auto reads_tag, const uint16_t* ra, const uint16_t* rb,
-                        int rkk, int lt, int ls, auto share_tag) __attribute__((always_inline)) {
+                        int rkk, int lt, int ls, auto share_tag, int ckk) __attribute__((always_inline)) {
     constexpr int kMi = decltype(mi_tag)::value;
     constexpr bool kDoReads = decltype(reads_tag)::value;
     constexpr int kMfmaEff = kMi * C::NJ, kReadsEff = kMi + C::NJ;
@@ -720,6 +757,15 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     constexpr int kShare = decltype(share_tag)::value;
     constexpr int kL0 = kShare * kLoads / C::KK;
     constexpr int kLn = (kShare + 1) * kLoads / C::KK - kL0;
+    if constexpr (kRagK) {
+      // a phase's last K step: the A fragments of contraction indices behind its end are zero
+      if (ckk >= 0) {
+        const bool dead = 16 * ckk + 8 * kc_piece >= k_rem;
+        const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < kMi; ++i) fa[par][i] = dead ? zero : fa[par][i];
+      }
+    }
     static_for<kMfmaEff>([&](auto mc) __attribute__((always_inline)) {
       constexpr int m = decltype(mc)::value;
       if constexpr (kDoReads) {
@@ -755,10 +801,15 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
     const uint16_t* na = lds + nxt * kStageElems;
     const uint16_t* nb = na + C::A_ELEMS;
     constexpr int kLoads = a_chunks_needed<C>(decltype(mi_tag)::value) + C::B_CHUNKS;
+    bool partial = false;
+    if constexpr (kRagK) {
+      const int in_phase = (kMode == kNTUpGate && kt >= kt_per_phase) ? kt - kt_per_phase : kt;
+      partial = in_phase == kt_per_phase - 1;
+    }
     static_for<C::KK - 1>([&](auto kc) __attribute__((always_inline)) {
       constexpr int kk = decltype(kc)::value;
       mfma_block(mi_tag, kk & 1, std::true_type{}, sa, sb, kk + 1, kt + S - 1, prv,
-                 std::integral_constant<int, kk + 1>{});
+                 std::integral_constant<int, kk + 1>{}, partial ? kk : -1);
     });
     if constexpr (kNext) {
       // Step kt+1 has landed once only the later steps' instructions are
@@ -768,10 +819,10 @@ __global__ __launch_bounds__(C::THREADS, C::OCC) void grouped_gemm_dma_kernel(Ge
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
       mfma_block(mi_tag, (C::KK - 1) & 1, std::true_type{}, na, nb, 0, kt + S, cur,
-                 std::integral_constant<int, 0>{});
+                 std::integral_constant<int, 0>{}, partial ? C::KK - 1 : -1);
     } else {
       mfma_block(mi_tag, (C::KK - 1) & 1, std::false_type{}, na, nb, 0, kt + S, cur,
-                 std::integral_constant<int, 0>{});
+                 std::integral_constant<int, 0>{}, partial ? C::KK - 1 : -1);
     }
   };
 
@@ -1382,8 +1433,12 @@ using WgradPers = DmaCfg<256, 256, 32, 2, 2, 3>;  // persistent weight gradient
 unsigned long long* g_clock_sink = nullptr;
 #endif
 
-template <typename C, int kMode>
+template <typename C, int kMode, bool kRagK = false>
 int launch_rows_dma(GemmParams p, int table_kind, int64_t rows_pad, int32_t num_banks, void* stream) {
+  if constexpr (!kRagK) {
+    // a contraction that ends inside a K step takes the variant that handles it
+    if (p.K % C::BK != 0) return launch_rows_dma<C, kMode, true>(p, table_kind, rows_pad, num_banks, stream);
+  }
   static_assert(C::BM == 128 || C::BM == 160 || C::BM == 320, "a tile table exists for these heights");
   if (32 * tile_blocks_cap(table_kind) > C::BM) return NESTOR_HIP_EINVAL;
   p.tile_table += table_offset(table_kind, rows_pad, num_banks);
@@ -1405,9 +1460,9 @@ int launch_rows_dma(GemmParams p, int table_kind, int64_t rows_pad, int32_t num_
   const int64_t blocks = ceil_div(p.max_tiles, gran) * gran * p.n_tiles;
   if (blocks > INT32_MAX) return NESTOR_HIP_ERANGE;
   static const bool configured = allow_dynamic_lds(
-      reinterpret_cast<const void*>(grouped_gemm_dma_kernel<C, kMode>), C::LDS_BYTES);
+      reinterpret_cast<const void*>(grouped_gemm_dma_kernel<C, kMode, kRagK>), C::LDS_BYTES);
   (void)configured;
-  hipLaunchKernelGGL((grouped_gemm_dma_kernel<C, kMode>), dim3(static_cast<unsigned>(blocks)),
+  hipLaunchKernelGGL((grouped_gemm_dma_kernel<C, kMode, kRagK>), dim3(static_cast<unsigned>(blocks)),
                      dim3(C::THREADS), C::LDS_BYTES, static_cast<hipStream_t>(stream), p);
   return launch_status();
 }
@@ -1425,8 +1480,8 @@ int dispatch_rows_gemm(const GemmParams& p, int64_t rows_pad, int32_t num_banks,
     // with one row of wavefronts (cfg 3).  The input-gradient GEMMs (both operands
     // contraction-contiguous, so every transfer is made of 64-byte row pieces) prefer
     // x256x32 with 2 x 2 wavefronts (cfg 7), which moves 20 % fewer pieces per MFMA.
-    // Narrower outputs take the x256x64 tile (cfg 4); a contraction that is not a
-    // multiple of the K step takes the register-staged kernel (cfg 2 and below).
+    // Narrower outputs take the x256x64 tile (cfg 4).  The register-staged kernels
+    // (cfg 2 and below) remain for outputs narrower than 256 and operands of 4 GiB.
     cfg = kBContigMode ? 7 : 3;
     if (cfg == 3 && width < 512) cfg = 4;
   }
@@ -1435,11 +1490,11 @@ int dispatch_rows_gemm(const GemmParams& p, int64_t rows_pad, int32_t num_banks,
     // operand (and inside a tile's rows of activations) that fit 32 bits.
     const int64_t b_span = (kBContigMode ? p.N : p.K) * p.ldb * 2;
     const bool spans_fit = b_span < (int64_t{1} << 32) && 512 * p.lda * 2 < (int64_t{1} << 32);
-    if (spans_fit && cfg == 7 && width >= 256 && p.K % 32 == 0)
+    if (spans_fit && cfg == 7 && width >= 256)
       return launch_rows_dma<DmaSquare, kMode>(p, kTilesBal320, rows_pad, num_banks, stream);
-    if (spans_fit && (cfg == 3 || cfg == 7) && width >= 512 && p.K % 32 == 0)
+    if (spans_fit && (cfg == 3 || cfg == 7) && width >= 512)
       return launch_rows_dma<DmaXWide, kMode>(p, kTilesBal160, rows_pad, num_banks, stream);
-    if (spans_fit && cfg >= 3 && width >= 256 && p.K % 64 == 0)
+    if (spans_fit && cfg >= 3 && width >= 256)
       return launch_rows_dma<DmaWide, kMode>(p, kTiles128, rows_pad, num_banks, stream);
   }
   if (cfg >= 3) cfg = 2;

@@ -35,8 +35,8 @@ void check_rows(int64_t K, int64_t N, int64_t lda, int64_t ldb, int nrows, int64
   constexpr int A_CHUNKS = A_ROWS * BK / 8 / THREADS, B_CHUNKS = BN * BK / 8 / THREADS;
   constexpr int BW = BN / kSub;
   const int last_row = nrows - 1;
-  const int num_kt = static_cast<int>(K / BK);       // per phase (the B operand's walk)
-  const int num_kt_a = num_kt * phases;              // the A operand walks all phases
+  const int num_kt = static_cast<int>((K + BK - 1) / BK);  // per phase; the last one may be partial
+  const int k_rem = static_cast<int>(K % BK);              // valid contraction indices of a partial last step
   std::vector<int> filled(A_ROWS * BK / 8 + BN * BK / 8, 0);
   for (int wave = 0; wave < WAVES; ++wave)
     for (int lane = 0; lane < 64; ++lane) {
@@ -45,33 +45,43 @@ void check_rows(int64_t K, int64_t N, int64_t lda, int64_t ldb, int nrows, int64
         REQUIRE(ci < A_ROWS * BK / 8, "A stage position %d", ci);
         ++filled[ci];
         const uint32_t off = a_lane_offset<BK>(ci, last_row, lda);
-        for (int kt = 0; kt < num_kt_a; ++kt) {
-          // bytes from the tile's first row: the piece must lie in rows [0, nrows), columns [0, K)
-          const int64_t b0 = static_cast<int64_t>(kt) * BK * 2 + off;
-          const int64_t row = b0 / (lda * 2), col = (b0 % (lda * 2)) / 2;
-          REQUIRE(row >= 0 && row < nrows, "A row %ld of %d (wave %d lane %d i %d)", (long)row, nrows, wave, lane, i);
-          REQUIRE(col + 8 <= K * phases, "A columns %ld..+8 of %ld", (long)col, (long)(K * phases));
-        }
+        const uint32_t adj = k_rem ? kc_partial_adjust<BK>(ci, k_rem) : 0u;
+        REQUIRE(adj <= off, "A adjustment %u beyond the offset %u", adj, off);
+        for (int phase = 0; phase < phases; ++phase)
+          for (int kt = 0; kt < num_kt; ++kt) {
+            const bool part = k_rem != 0 && kt == num_kt - 1;
+            // bytes from the tile's first row: the piece must lie in rows [0, nrows) and in the
+            // phase's own K columns (the phases sit side by side in a row)
+            const int64_t b0 = static_cast<int64_t>(phase) * K * 2 + static_cast<int64_t>(kt) * BK * 2 + off - (part ? adj : 0);
+            const int64_t row = b0 / (lda * 2), col = (b0 % (lda * 2)) / 2;
+            REQUIRE(row >= 0 && row < nrows, "A row %ld of %d (wave %d lane %d i %d)", (long)row, nrows, wave, lane, i);
+            REQUIRE(col >= phase * K && col + 8 <= (phase + 1) * K, "A columns %ld..+8 of phase %d, K %ld", (long)col, phase, (long)K);
+          }
       }
       for (int i = 0; i < B_CHUNKS; ++i) {
         const int ci = (wave + WAVES * i) * 64 + lane;
         REQUIRE(ci < BN * BK / 8, "B stage position %d", ci);
         ++filled[A_ROWS * BK / 8 + ci];
         for (int kt = 0; kt < num_kt; ++kt) {
+          const bool part = k_rem != 0 && kt == num_kt - 1;
           if (kBContig) {
             // b is [N, K] (ldb elements per row): rows n0 .. N - 1, columns of K step kt
             const uint32_t off = b_contig_lane_offset<BK>(ci, n0, N, ldb);
-            const int64_t b0 = n0 * ldb * 2 + static_cast<int64_t>(kt) * BK * 2 + off;
+            const uint32_t adj = part ? kc_partial_adjust<BK>(ci, k_rem) : 0u;
+            REQUIRE(adj <= off, "B adjustment beyond the offset");
+            const int64_t b0 = n0 * ldb * 2 + static_cast<int64_t>(kt) * BK * 2 + off - adj;
             const int64_t row = b0 / (ldb * 2), col = (b0 % (ldb * 2)) / 2;
             REQUIRE(row >= n0 && row < N, "B row %ld of [%ld, %ld)", (long)row, (long)n0, (long)N);
             REQUIRE(col + 8 <= K, "B columns %ld..+8 of %ld", (long)col, (long)K);
           } else {
             // b is [K, N]: contraction rows of K step kt, columns n0 .. N - 1
             const uint32_t off = b_major_lane_offset<BK, BW>(ci, n0, N, ldb);
-            const int64_t b0 = n0 * 2 + static_cast<int64_t>(kt) * BK * ldb * 2 + off;
+            const uint32_t adj = part ? b_major_partial_adjust<BK, BW>(ci, k_rem, ldb) : 0u;
+            REQUIRE(adj <= off, "B adjustment beyond the offset");
+            const int64_t b0 = n0 * 2 + static_cast<int64_t>(kt) * BK * ldb * 2 + off - adj;
             const int64_t row = b0 / (ldb * 2), col = (b0 % (ldb * 2)) / 2;
             REQUIRE(row >= static_cast<int64_t>(kt) * BK && row < static_cast<int64_t>(kt + 1) * BK && row < K,
-                    "B contraction row %ld in step %d", (long)row, kt);
+                    "B contraction row %ld in step %d of K %ld", (long)row, kt, (long)K);
             REQUIRE(col >= 0 && col + 8 <= N, "B columns %ld..+8 of %ld (n0 %ld)", (long)col, (long)N, (long)n0);
           }
         }
@@ -138,6 +148,16 @@ int main() {
         check_rows<128, 256, 64, 4, true, 1>(1280, N, 1280, 1280, nrows, n0, 1);
         check_rows<128, 256, 64, 4, false, 1>(1280, N, 1280, N, nrows, n0, 1);
       }
+  // contractions that end inside a K step (the production widths 424, 216, 184; the shortest ones)
+  for (int64_t K : {8, 24, 40, 184, 216, 424})
+    for (int nrows : {1, 100, 160}) {
+      check_rows<160, 512, 32, 4, false, 1>(K, 1280, K, 1280, nrows, 0, 1);       // down projection, K = h
+      check_rows<160, 512, 32, 4, false, 1>(K, 1280, K, 1280, nrows, 1024, 1);
+      check_rows<320, 256, 32, 4, true, 1>(K, 1280, 2 * K, K, nrows, 1024, 2);    // fused up|gate input gradient, K = h
+      check_rows<320, 256, 32, 4, true, 1>(K, 424, K, K, nrows, 256, 1);
+      check_rows<128, 256, 64, 4, true, 1>(K, 320, 2 * K, K, nrows, 256, 2);
+      check_rows<128, 256, 64, 4, false, 2>(K, 160, K, 160, nrows, 128, 1);
+    }
   // weight gradient: segments whose length is not a multiple of the K step, operands narrower
   // than a tile, overhanging column tiles, the last segment ending with the operand
   for (int seg_rows : {1, 2, 16, 31, 32, 33, 100, 512, 530})

@@ -43,6 +43,13 @@ SHAPES = [
     # output dimensions, empty banks and segments of a few rows
     (1200, 2, 24, 264, 520, True),
     (40, 1, 12, 256, 256, True),
+    # contractions that end inside a K step on the direct-to-LDS path (the production
+    # widths): forward with K = 424 / 216 / 8, input gradient with K = 424 / 184
+    (1500, 2, 6, 424, 1280, False),
+    (1500, 2, 6, 1280, 424, True),
+    (900, 3, 5, 216, 640, False),
+    (640, 1, 3, 8, 512, False),
+    (1100, 2, 4, 640, 184, False),
 ]
 
 
@@ -78,6 +85,9 @@ def test_segment_mm_forward_and_grads(cuda, tokens, slots, banks, K, N, skew):
     (300, 2, 6, 40, 24, False), (1000, 3, 20, 512, 1024, False), (700, 2, 16, 200, 424, True),
     (2048, 1, 4, 1024, 2048, False),
     (500, 2, 5, 64, 256, False), (600, 1, 4, 96, 520, False), (900, 2, 6, 512, 576, True),
+    # production widths: the fused input gradient contracts over 2 x 424 / 2 x 216 columns,
+    # each phase ending inside a K step
+    (1500, 2, 6, 1280, 424, False), (900, 3, 5, 640, 216, True), (700, 2, 4, 200, 184, False),
 ])
 def test_upgate_swiglu_fused_matches_unfused(cuda, tokens, slots, banks, K, H, skew):
     """The fused up|gate + SwiGLU kernel against the oracle chain with the
