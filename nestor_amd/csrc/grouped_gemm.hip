@@ -1483,7 +1483,10 @@ int dispatch_rows_gemm(const GemmParams& p, int64_t rows_pad, int32_t num_banks,
     // Narrower outputs take the x256x64 tile (cfg 4).  The register-staged kernels
     // (cfg 2 and below) remain for outputs narrower than 256 and operands of 4 GiB.
     cfg = kBContigMode ? 7 : 3;
-    if (cfg == 3 && width < 512) cfg = 4;
+    // The fused up|gate tile holds 256 up and 256 gate columns: from 129 columns of each on
+    // it beats two passes of the 128 + 128 tile over the activations (measured at h = 160,
+    // 184, 216: 15-24 % faster), although up to half of its weight panel is padding.
+    if (cfg == 3 && width < (kMode == kNNUpGate ? 264 : 512)) cfg = 4;
   }
   if constexpr (kMode != kNNFp8W) {
     // Direct-to-LDS variants: whole K steps only, and byte offsets inside one bank's
@@ -1492,7 +1495,7 @@ int dispatch_rows_gemm(const GemmParams& p, int64_t rows_pad, int32_t num_banks,
     const bool spans_fit = b_span < (int64_t{1} << 32) && 512 * p.lda * 2 < (int64_t{1} << 32);
     if (spans_fit && cfg == 7 && width >= 256)
       return launch_rows_dma<DmaSquare, kMode>(p, kTilesBal320, rows_pad, num_banks, stream);
-    if (spans_fit && (cfg == 3 || cfg == 7) && width >= 512)
+    if (spans_fit && (cfg == 3 || cfg == 7) && width >= 264)
       return launch_rows_dma<DmaXWide, kMode>(p, kTilesBal160, rows_pad, num_banks, stream);
     if (spans_fit && cfg >= 3 && width >= 256)
       return launch_rows_dma<DmaWide, kMode>(p, kTiles128, rows_pad, num_banks, stream);
@@ -1654,10 +1657,13 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
   p.seg_start = seg_start;
   p.seg_count = seg_count;
   static const int forced = config_choice("NESTOR_HIP_WGRAD_CFG", -1);
-  int cfg = forced >= 0 ? forced : ((M >= 256 && N >= 256) ? 5 : 0);
+  // The persistent kernel's 256 x 256 tiles may overhang the outputs: it wins from 128
+  // columns on (1280 x 160 outputs: 0.31 -> 0.21 ms; its descriptors cut the overhang off).
+  static const int pers_min = config_choice("NESTOR_HIP_WGRAD_MIN", 128);
+  int cfg = forced >= 0 ? forced : ((M >= pers_min && N >= pers_min) ? 5 : 0);
   // the persistent kernel's buffer descriptors count an operand's bytes in 32 bits
   const bool spans_fit = rows_pad * lda * 2 < (int64_t{1} << 32) && rows_pad * ldg * 2 < (int64_t{1} << 32);
-  if (cfg == 5 && M >= 256 && N >= 256 && rows_pad <= INT32_MAX && spans_fit) {
+  if (cfg == 5 && M >= pers_min && N >= pers_min && rows_pad <= INT32_MAX && spans_fit) {
     using C = WgradPers;
     static const bool configured =
         allow_dynamic_lds(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, false>),

@@ -161,7 +161,7 @@ int main() {
   // weight gradient: segments whose length is not a multiple of the K step, operands narrower
   // than a tile, overhanging column tiles, the last segment ending with the operand
   for (int seg_rows : {1, 2, 16, 31, 32, 33, 100, 512, 530})
-    for (int64_t cols : {256, 264, 424, 2048})
+    for (int64_t cols : {64, 160, 216, 256, 264, 424, 2048})
       for (int64_t ld : {cols, cols + 8, 2 * cols})
         for (int m0 = 0; m0 < cols; m0 += 256) {
           check_wgrad(seg_rows, 0, seg_rows, ld, cols, m0);                 // the operand is this segment
