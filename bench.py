@@ -196,9 +196,9 @@ def bank_call_breakdown(x, grad_out, ids, weights, bank3, iters: int = 5,
          2.0 * rows * d * 2 * h)
     gx_pad = ops.grouped_gemm_nt_upgate(gug, w_up, w_gate, plan.tile_table)
 
-    gemm("gemm_wgrad_up(one of 2)",
-         lambda: ops.grouped_gemm_tn(x_pad, gug[:, :h], plan.offs, plan.padded_starts, plan.counts),
-         2.0 * rows * d * h)
+    gemm("gemm_wgrad_upgate_pair",
+         lambda: ops.grouped_gemm_tn_pair(x_pad, gug, plan.offs, plan.padded_starts, plan.counts),
+         2.0 * rows * d * 2 * h)
     if gemms_only:
         return out
 

@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define NESTOR_HIP_ABI_VERSION 15
+#define NESTOR_HIP_ABI_VERSION 16
 
 /* status codes */
 #define NESTOR_HIP_OK 0
@@ -284,6 +284,20 @@ int nestor_hip_grouped_gemm_nt_upgate(
 int nestor_hip_grouped_gemm_tn(
     const void* a, int64_t lda, const void* g, int64_t ldg,
     void* out, int64_t ldo, int64_t bank_stride,
+    int64_t rows_pad, int64_t M, int64_t N, int32_t num_banks,
+    const int32_t* offs, const int64_t* seg_start, const int64_t* seg_count,
+    int32_t out_dtype, void* stream);
+
+/* The two weight gradients of the fused up|gate GEMM in one call: g [rows_pad, 2N] holds
+ * the gradient of the up columns, then of the gate columns (the backward of
+ * grouped_mm_fused_gate's concatenated weight, nestor/backbones/triton_expert.py:444-453
+ * splits one [E,d,2h] gradient into the two owners'); out0[e] = a_seg^T @ g_seg[:, :N],
+ * out1[e] = a_seg^T @ g_seg[:, N:], both [E,M,N] with the same strides and dtype.  One
+ * launch when N is a multiple of 256 (the gradients share the activation panels), else
+ * two nestor_hip_grouped_gemm_tn launches; the results are the same bits either way. */
+int nestor_hip_grouped_gemm_tn_pair(
+    const void* a, int64_t lda, const void* g, int64_t ldg,
+    void* out0, void* out1, int64_t ldo, int64_t bank_stride,
     int64_t rows_pad, int64_t M, int64_t N, int32_t num_banks,
     const int32_t* offs, const int64_t* seg_start, const int64_t* seg_count,
     int32_t out_dtype, void* stream);

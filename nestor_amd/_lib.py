@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_int32, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libnestor_hip.so"
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 F32 = 0
 BF16 = 1
@@ -66,6 +66,9 @@ _SIGNATURES: dict[str, list] = {
     ],
     "nestor_hip_grouped_gemm_tn": [
         _P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _I32, _P, _P, _P, _I32, _P,
+    ],
+    "nestor_hip_grouped_gemm_tn_pair": [
+        _P, _I64, _P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I64, _I32, _P, _P, _P, _I32, _P,
     ],
     "nestor_hip_grouped_gemm_fp8w_nn": [_P, _P, _P, _P, _I64, _I64, _I64, _I32, _P, _I64, _I32, _P],
     "nestor_hip_grouped_gemm_fp8w_upgate_swiglu": [

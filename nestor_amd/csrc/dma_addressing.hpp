@@ -80,11 +80,13 @@ NESTOR_HD uint32_t b_major_partial_adjust(int ci, int k_rem, int64_t ldb) {
 }
 
 // ---- persistent weight gradient ----------------------------------------------
-// Both operands are [segment row, column] with 256-column tiles: one transfer covers
-// two contraction rows x 32 pieces.
-NESTOR_HD uint32_t wgrad_lane_offset(int wave, int waves, int chunk, int lane, int64_t ld) {
-  const int krow = 2 * (wave + waves * chunk) + (lane >> 5);
-  const int pc = (lane & 31) ^ (4 * (krow & 3));
+// Both operands are [segment row, column] with tiles of 256 or 128 columns: one transfer
+// covers two contraction rows x 32 pieces, or four x 16.
+NESTOR_HD uint32_t wgrad_lane_offset(int wave, int waves, int chunk, int lane, int64_t ld,
+                                     int tile_cols = 256) {
+  const int ppr = tile_cols / 8;  // pieces per contraction row of the tile
+  const int krow = (64 / ppr) * (wave + waves * chunk) + lane / ppr;
+  const int pc = (lane % ppr) ^ (4 * (krow & 3));
   return static_cast<uint32_t>((static_cast<int64_t>(krow) * ld + pc * 8) * 2);
 }
 // num_records of the descriptor that starts at (segment row 0, column m0) of an

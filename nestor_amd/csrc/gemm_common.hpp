@@ -95,6 +95,7 @@ struct GemmParams {
   const int64_t* seg_start;
   const int64_t* seg_count;
   int out_f32;          // kTN: out is float* (fp32 results), not bf16
+  int64_t split;        // kTN pair: output columns from `split` on go to out2 (column - split); 0: one output
   // Measurement hook of the direct-to-LDS kernels (null in normal use): 64 slots of
   // {shader cycles, wall-clock ticks, workgroups, K steps}, summed over the
   // workgroups of a launch (slot = workgroup index % 64).

@@ -988,10 +988,12 @@ template <typename C>
 struct WgradLayout {
   static constexpr int kMaxItems = 1024;
   static constexpr int kRingElems = C::kStages * (C::A_ELEMS + C::B_ELEMS);
-  static constexpr int kEpiLd = C::WTN + 8;
+  static constexpr int kEpiCols = C::WTN;  // bf16 columns of a slab
+  static constexpr int kEpiLd = kEpiCols + 8;
   static constexpr int kEpiElems = 32 * kEpiLd;  // one 32-row slab per wavefront
   static constexpr int kTableOffset = kRingElems + C::WAVES * kEpiElems;  // in uint16 units
   static constexpr size_t LDS_BYTES = sizeof(uint16_t) * kTableOffset + 16 * kMaxItems;
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS of one CU");
 };
 
 // kOutF32: the gradient tile leaves as fp32 straight from the accumulators (no bf16
@@ -1094,9 +1096,9 @@ __global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmPar
   static_assert(BM / 8 == 32 && BN / 8 == 32, "one DMA instruction covers two contraction rows");
   uint32_t offa[C::A_CHUNKS], offb[C::B_CHUNKS];
 #pragma unroll
-  for (int c = 0; c < C::A_CHUNKS; ++c) offa[c] = dma::wgrad_lane_offset(wave, kWaves, c, lane, p.lda);
+  for (int c = 0; c < C::A_CHUNKS; ++c) offa[c] = dma::wgrad_lane_offset(wave, kWaves, c, lane, p.lda, BM);
 #pragma unroll
-  for (int c = 0; c < C::B_CHUNKS; ++c) offb[c] = dma::wgrad_lane_offset(wave, kWaves, c, lane, p.ldb);
+  for (int c = 0; c < C::B_CHUNKS; ++c) offb[c] = dma::wgrad_lane_offset(wave, kWaves, c, lane, p.ldb, BN);
   i32x4 desc_a = buffer_descriptor(p.a, 0), desc_b = buffer_descriptor(p.b0, 0);
   // bytes per K step; the launcher checks that a whole operand spans less than 4 GiB
   const uint32_t step_a = static_cast<uint32_t>(BK * p.lda * 2), step_b = static_cast<uint32_t>(BK * p.ldb * 2);
@@ -1216,24 +1218,31 @@ __global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmPar
     const int nt = __builtin_amdgcn_readfirstlane(t.w);
     const int bank = rt / m_tiles;
     const int m0 = (rt - bank * m_tiles) * BM;
-    const int n0 = nt * BN;
+    // a pair launch (p.split > 0, a multiple of BN): the column tiles from `split` on belong
+    // to the second output
+    const bool second = p.split > 0 && static_cast<int64_t>(nt) * BN >= p.split;
+    const int n0 = nt * BN - (second ? static_cast<int>(p.split) : 0);
+    const int64_t n_end = p.split > 0 ? p.split : p.N;   // columns of one output
+    uint16_t* const out_base = second ? p.out2 : p.out;
     if constexpr (kOutF32) {
       // fp32 results through the same per-wavefront slab, half as many columns at a
       // time (32 rows x 64 columns of fp32 fill the space of 32 x 128 of bf16), so that
       // every store instruction still writes whole 256-byte row segments.  (Storing
       // each lane's four columns directly writes 32-byte pieces: 2.7x slower.)
-      float* out32 = reinterpret_cast<float*>(p.out) + bank * p.bank_stride;
+      float* out32 = reinterpret_cast<float*>(out_base) + bank * p.bank_stride;
       float* epi32 = reinterpret_cast<float*>(epi);
-      constexpr int kLd32 = L::kEpiLd / 2;  // floats per slab row: 64 + 4 of padding
-      static_assert(L::kEpiLd % 2 == 0 && kLd32 >= 64 + 4, "slab row holds 64 floats");
-      static_assert(C::NJ % 2 == 0, "column blocks are staged in pairs");
+      constexpr int kCols32 = L::kEpiCols / 2;  // fp32 columns per pass
+      constexpr int kBlk32 = kCols32 / 32;      // column blocks per pass
+      constexpr int kLd32 = L::kEpiLd / 2;      // floats per slab row: kCols32 + 4 of padding
+      static_assert(L::kEpiLd % 2 == 0 && kLd32 >= kCols32 + 4, "slab row holds a pass's floats");
+      static_assert(C::NJ % kBlk32 == 0, "whole passes");
 #pragma unroll
       for (int i = 0; i < C::MI; ++i)
 #pragma unroll
-        for (int jp = 0; jp < C::NJ / 2; ++jp) {
+        for (int jp = 0; jp < C::NJ / kBlk32; ++jp) {
           __builtin_amdgcn_sched_barrier(0);  // one slab's worth of registers at a time
 #pragma unroll
-          for (int jj = 0; jj < 2; ++jj)
+          for (int jj = 0; jj < kBlk32; ++jj)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               f32x4 v;
@@ -1241,64 +1250,68 @@ __global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmPar
               for (int e = 0; e < 4; ++e)
                 asm volatile("v_accvgpr_read_b32 %0, %1"
                              : "=v"(v[e])
-                             : "a"(acc[i][2 * jp + jj][4 * q + e]));
+                             : "a"(acc[i][kBlk32 * jp + jj][4 * q + e]));
               *reinterpret_cast<f32x4*>(epi32 + (lane & 31) * kLd32 + 32 * jj + 8 * q +
                                         4 * (lane >> 5)) = v;
             }
-          constexpr int kPieces32 = 32 * 16 / 64;  // 16-byte pieces per lane
+          constexpr int kCpr32 = kCols32 / 4;         // 16-byte pieces per slab row
+          constexpr int kPieces32 = 32 * kCpr32 / 64;  // per lane
           f32x4 piece[kPieces32];
 #pragma unroll
           for (int t = 0; t < kPieces32; ++t) {
             const int c = lane + 64 * t;
-            piece[t] = *reinterpret_cast<const f32x4*>(epi32 + (c / 16) * kLd32 + (c % 16) * 4);
+            piece[t] = *reinterpret_cast<const f32x4*>(epi32 + (c / kCpr32) * kLd32 + (c % kCpr32) * 4);
           }
 #pragma unroll
           for (int t = 0; t < kPieces32; ++t) {
             const int c = lane + 64 * t;
-            const int64_t m = m0 + C::WTM * wm + 32 * i + c / 16;
-            const int64_t n = n0 + C::WTN * wn + 64 * jp + (c % 16) * 4;
-            if (m < p.M && n < p.N)
+            const int64_t m = m0 + C::WTM * wm + 32 * i + c / kCpr32;
+            const int64_t n = n0 + C::WTN * wn + kCols32 * jp + (c % kCpr32) * 4;
+            if (m < p.M && n < n_end)
               __builtin_nontemporal_store(piece[t], reinterpret_cast<f32x4*>(out32 + m * p.ldo + n));
           }
         }
       return;
     }
-    uint16_t* out = p.out + bank * p.bank_stride;
+    uint16_t* out = out_base + bank * p.bank_stride;
+    constexpr int kBlk = L::kEpiCols / 32;  // column blocks per pass
 #pragma unroll
-    for (int i = 0; i < C::MI; ++i) {
-      __builtin_amdgcn_sched_barrier(0);  // one slab's worth of registers at a time
+    for (int i = 0; i < C::MI; ++i)
 #pragma unroll
-      for (int j = 0; j < C::NJ; ++j)
+      for (int jg = 0; jg < C::NJ / kBlk; ++jg) {
+        __builtin_amdgcn_sched_barrier(0);  // one slab's worth of registers at a time
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = 32 * j + 8 * q + 4 * (lane >> 5);
-          // Read the accumulators where they are used: left to the compiler, all
-          // 256 reads move to the top of the epilogue and spill.
-          float v[4];
+        for (int jj = 0; jj < kBlk; ++jj)
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][j][4 * q + e]));
-          u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-          *reinterpret_cast<u32x2*>(epi + (lane & 31) * L::kEpiLd + n) = packed;
+          for (int q = 0; q < 4; ++q) {
+            const int n = 32 * jj + 8 * q + 4 * (lane >> 5);
+            // Read the accumulators where they are used: left to the compiler, all
+            // 256 reads move to the top of the epilogue and spill.
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i][kBlk * jg + jj][4 * q + e]));
+            u32x2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            *reinterpret_cast<u32x2*>(epi + (lane & 31) * L::kEpiLd + n) = packed;
+          }
+        // The same wavefront wrote and reads: program order is enough.  All reads
+        // go out before the first store so that their latencies overlap.
+        constexpr int kCpr = L::kEpiCols / 8;
+        constexpr int kPieces = 32 * kCpr / 64;
+        u32x4 piece[kPieces];
+#pragma unroll
+        for (int t = 0; t < kPieces; ++t) {
+          const int c = lane + 64 * t;
+          piece[t] = *reinterpret_cast<const u32x4*>(epi + (c / kCpr) * L::kEpiLd + (c % kCpr) * 8);
         }
-      // The same wavefront wrote and reads: program order is enough.  All reads
-      // go out before the first store so that their latencies overlap.
-      constexpr int kCpr = C::WTN / 8;
-      constexpr int kPieces = 32 * kCpr / 64;
-      u32x4 piece[kPieces];
 #pragma unroll
-      for (int t = 0; t < kPieces; ++t) {
-        const int c = lane + 64 * t;
-        piece[t] = *reinterpret_cast<const u32x4*>(epi + (c / kCpr) * L::kEpiLd + (c % kCpr) * 8);
+        for (int t = 0; t < kPieces; ++t) {
+          const int c = lane + 64 * t;
+          const int64_t m = m0 + C::WTM * wm + 32 * i + c / kCpr;
+          const int64_t n = n0 + C::WTN * wn + L::kEpiCols * jg + (c % kCpr) * 8;
+          if (m < p.M && n < n_end) st16o(out + m * p.ldo + n, piece[t]);
+        }
       }
-#pragma unroll
-      for (int t = 0; t < kPieces; ++t) {
-        const int c = lane + 64 * t;
-        const int64_t m = m0 + C::WTM * wm + 32 * i + c / kCpr;
-        const int64_t n = n0 + C::WTN * wn + (c % kCpr) * 8;
-        if (m < p.M && n < p.N) st16o(out + m * p.ldo + n, piece[t]);
-      }
-    }
   };
   // This wavefront's part of an output tile whose bank has no rows.
   auto store_zero_tile = [&](int item) __attribute__((always_inline)) {
@@ -1307,19 +1320,22 @@ __global__ __launch_bounds__(C::THREADS, 1) void wgrad_persistent_kernel(GemmPar
     const int nt = __builtin_amdgcn_readfirstlane(t.w);
     const int bank = rt / m_tiles;
     const int m0 = (rt - bank * m_tiles) * BM;
-    const int n0 = nt * BN;
+    const bool second = p.split > 0 && static_cast<int64_t>(nt) * BN >= p.split;
+    const int n0 = nt * BN - (second ? static_cast<int>(p.split) : 0);
+    const int64_t n_end = p.split > 0 ? p.split : p.N;
+    uint16_t* const out_base = second ? p.out2 : p.out;
     constexpr int kCpr = C::WTN / 8;
     const u32x4 zero = {0, 0, 0, 0};
     for (int c = lane; c < C::WTM * kCpr; c += 64) {
       const int64_t m = m0 + C::WTM * wm + c / kCpr;
       const int64_t n = n0 + C::WTN * wn + (c % kCpr) * 8;
-      if (m < p.M && n < p.N) {
+      if (m < p.M && n < n_end) {
         if constexpr (kOutF32) {
-          float* o = reinterpret_cast<float*>(p.out) + bank * p.bank_stride + m * p.ldo + n;
+          float* o = reinterpret_cast<float*>(out_base) + bank * p.bank_stride + m * p.ldo + n;
           st16o(o, zero);
           st16o(o + 4, zero);
         } else {
-          st16o(p.out + bank * p.bank_stride + m * p.ldo + n, zero);
+          st16o(out_base + bank * p.bank_stride + m * p.ldo + n, zero);
         }
       }
     }
@@ -1627,20 +1643,75 @@ extern "C" int nestor_hip_grouped_gemm_nt_upgate(
   return dispatch_rows_gemm<kNTUpGate>(p, rows_pad, num_banks, stream);
 }
 
-extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void* g,
-                                          int64_t ldg, void* out, int64_t ldo,
-                                          int64_t bank_stride, int64_t rows_pad, int64_t M,
-                                          int64_t N, int32_t num_banks, const int32_t* offs,
-                                          const int64_t* seg_start, const int64_t* seg_count,
-                                          int32_t out_dtype, void* stream) {
+namespace nestor {
+namespace {
+
+bool tn_args_ok(const void* a, int64_t lda, const void* g, int64_t ldg, const void* out, int64_t ldo,
+                int64_t rows_pad, int64_t M, int64_t N, int64_t g_cols, int32_t num_banks,
+                const int32_t* offs, const int64_t* seg_start, const int64_t* seg_count,
+                int32_t out_dtype) {
   if (rows_pad < 0 || M <= 0 || N <= 0 || M % 8 != 0 || N % 8 != 0 || lda % 8 != 0 ||
-      ldg % 8 != 0 || ldo % 8 != 0 || lda < M || ldg < N || ldo < N || num_banks <= 0 ||
+      ldg % 8 != 0 || ldo % 8 != 0 || lda < M || ldg < g_cols || ldo < N || num_banks <= 0 ||
       num_banks > 65535)
-    return NESTOR_HIP_EINVAL;
-  if (!out || (!offs && !(seg_start && seg_count)) || (rows_pad > 0 && (!a || !g)))
-    return NESTOR_HIP_EINVAL;
-  if ((seg_start == nullptr) != (seg_count == nullptr)) return NESTOR_HIP_EINVAL;
-  if (out_dtype != NESTOR_HIP_BF16 && out_dtype != NESTOR_HIP_F32) return NESTOR_HIP_EINVAL;
+    return false;
+  if (!out || (!offs && !(seg_start && seg_count)) || (rows_pad > 0 && (!a || !g))) return false;
+  if ((seg_start == nullptr) != (seg_count == nullptr)) return false;
+  return out_dtype == NESTOR_HIP_BF16 || out_dtype == NESTOR_HIP_F32;
+}
+
+// The persistent kernel when the shape allows it (returns 1 when it does not), else a status.
+int launch_wgrad_persistent(GemmParams p, int32_t num_banks, void* stream) {
+  using C = WgradPers;
+  // its buffer descriptors count an operand's bytes in 32 bits
+  const bool spans_fit =
+      p.rows_pad * p.lda * 2 < (int64_t{1} << 32) && p.rows_pad * p.ldb * 2 < (int64_t{1} << 32);
+  if (p.rows_pad > INT32_MAX || !spans_fit) return 1;
+  static const bool configured =
+      allow_dynamic_lds(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, false>),
+                        WgradLayout<C>::LDS_BYTES) &&
+      allow_dynamic_lds(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, true>),
+                        WgradLayout<C>::LDS_BYTES);
+  (void)configured;
+  const int num_cus = cu_count() / 8 * 8;
+  const int64_t items = ceil_div(p.M, C::BM) * ceil_div(p.N, C::BN) * num_banks;
+  if (num_cus < 8 || items / num_cus + 2 > WgradLayout<C>::kMaxItems) return 1;
+#if NESTOR_GEMM_CLOCK_HOOK
+  p.clock_sink = g_clock_sink;
+#endif
+  if (p.out_f32)
+    hipLaunchKernelGGL((wgrad_persistent_kernel<C, true>), dim3(static_cast<unsigned>(num_cus)),
+                       dim3(C::THREADS), WgradLayout<C>::LDS_BYTES,
+                       static_cast<hipStream_t>(stream), p, num_banks);
+  else
+    hipLaunchKernelGGL((wgrad_persistent_kernel<C, false>), dim3(static_cast<unsigned>(num_cus)),
+                       dim3(C::THREADS), WgradLayout<C>::LDS_BYTES,
+                       static_cast<hipStream_t>(stream), p, num_banks);
+  return launch_status();
+}
+
+// One weight gradient: which kernel takes it.
+int launch_tn(const GemmParams& p, int32_t num_banks, void* stream) {
+  static const int forced = config_choice("NESTOR_HIP_WGRAD_CFG", -1);
+  // The persistent kernel's 256 x 256 tiles may overhang the outputs: it wins from 128
+  // columns on (1280 x 160 outputs: 0.31 -> 0.21 ms; its descriptors cut the overhang off).
+  static const int pers_min = config_choice("NESTOR_HIP_WGRAD_MIN", 128);
+  int cfg = forced >= 0 ? forced : ((p.M >= pers_min && p.N >= pers_min) ? 5 : 0);
+  if (cfg == 5 && p.M >= pers_min && p.N >= pers_min) {
+    const int rc = launch_wgrad_persistent(p, num_banks, stream);
+    if (rc <= 0) return rc;
+  }
+  if (cfg == 5) cfg = 3;
+  switch (cfg) {
+    case 3: return launch_wgrad<CfgSquare>(p, num_banks, stream);
+    case 1: return launch_wgrad<CfgWide>(p, num_banks, stream);
+    default: return launch_wgrad<CfgSmall>(p, num_banks, stream);
+  }
+}
+
+GemmParams tn_params(const void* a, int64_t lda, const void* g, int64_t ldg, void* out, int64_t ldo,
+                     int64_t bank_stride, int64_t rows_pad, int64_t M, int64_t N,
+                     const int32_t* offs, const int64_t* seg_start, const int64_t* seg_count,
+                     int32_t out_dtype) {
   GemmParams p = {};
   p.out_f32 = out_dtype == NESTOR_HIP_F32;
   p.a = static_cast<const uint16_t*>(a);
@@ -1656,44 +1727,54 @@ extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void
   p.offs = offs;
   p.seg_start = seg_start;
   p.seg_count = seg_count;
+  return p;
+}
+
+}  // namespace
+}  // namespace nestor
+
+extern "C" int nestor_hip_grouped_gemm_tn(const void* a, int64_t lda, const void* g,
+                                          int64_t ldg, void* out, int64_t ldo,
+                                          int64_t bank_stride, int64_t rows_pad, int64_t M,
+                                          int64_t N, int32_t num_banks, const int32_t* offs,
+                                          const int64_t* seg_start, const int64_t* seg_count,
+                                          int32_t out_dtype, void* stream) {
+  if (!tn_args_ok(a, lda, g, ldg, out, ldo, rows_pad, M, N, N, num_banks, offs, seg_start, seg_count,
+                  out_dtype))
+    return NESTOR_HIP_EINVAL;
+  return launch_tn(tn_params(a, lda, g, ldg, out, ldo, bank_stride, rows_pad, M, N, offs, seg_start,
+                             seg_count, out_dtype),
+                   num_banks, stream);
+}
+
+extern "C" int nestor_hip_grouped_gemm_tn_pair(const void* a, int64_t lda, const void* g,
+                                               int64_t ldg, void* out0, void* out1, int64_t ldo,
+                                               int64_t bank_stride, int64_t rows_pad, int64_t M,
+                                               int64_t N, int32_t num_banks, const int32_t* offs,
+                                               const int64_t* seg_start, const int64_t* seg_count,
+                                               int32_t out_dtype, void* stream) {
+  if (!tn_args_ok(a, lda, g, ldg, out0, ldo, rows_pad, M, N, 2 * N, num_banks, offs, seg_start,
+                  seg_count, out_dtype) || !out1)
+    return NESTOR_HIP_EINVAL;
+  GemmParams p = tn_params(a, lda, g, ldg, out0, ldo, bank_stride, rows_pad, M, N, offs, seg_start,
+                           seg_count, out_dtype);
   static const int forced = config_choice("NESTOR_HIP_WGRAD_CFG", -1);
-  // The persistent kernel's 256 x 256 tiles may overhang the outputs: it wins from 128
-  // columns on (1280 x 160 outputs: 0.31 -> 0.21 ms; its descriptors cut the overhang off).
-  static const int pers_min = config_choice("NESTOR_HIP_WGRAD_MIN", 128);
-  int cfg = forced >= 0 ? forced : ((M >= pers_min && N >= pers_min) ? 5 : 0);
-  // the persistent kernel's buffer descriptors count an operand's bytes in 32 bits
-  const bool spans_fit = rows_pad * lda * 2 < (int64_t{1} << 32) && rows_pad * ldg * 2 < (int64_t{1} << 32);
-  if (cfg == 5 && M >= pers_min && N >= pers_min && rows_pad <= INT32_MAX && spans_fit) {
-    using C = WgradPers;
-    static const bool configured =
-        allow_dynamic_lds(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, false>),
-                          WgradLayout<C>::LDS_BYTES) &&
-        allow_dynamic_lds(reinterpret_cast<const void*>(wgrad_persistent_kernel<C, true>),
-                          WgradLayout<C>::LDS_BYTES);
-    (void)configured;
-    const int num_cus = cu_count() / 8 * 8;
-    const int64_t items = ceil_div(M, C::BM) * ceil_div(N, C::BN) * num_banks;
-    if (num_cus >= 8 && items / num_cus + 2 <= WgradLayout<C>::kMaxItems) {
-#if NESTOR_GEMM_CLOCK_HOOK
-      p.clock_sink = g_clock_sink;
-#endif
-      if (p.out_f32)
-        hipLaunchKernelGGL((wgrad_persistent_kernel<C, true>), dim3(static_cast<unsigned>(num_cus)),
-                           dim3(C::THREADS), WgradLayout<C>::LDS_BYTES,
-                           static_cast<hipStream_t>(stream), p, num_banks);
-      else
-        hipLaunchKernelGGL((wgrad_persistent_kernel<C, false>), dim3(static_cast<unsigned>(num_cus)),
-                           dim3(C::THREADS), WgradLayout<C>::LDS_BYTES,
-                           static_cast<hipStream_t>(stream), p, num_banks);
-      return launch_status();
-    }
+  static const bool pair_off = config_choice("NESTOR_HIP_WGRAD_PAIR", 1) == 0;
+  // One launch over both halves of g when a column tile never straddles them: the two
+  // gradients share the activation panels and one launch's ramp and tail.
+  if ((forced < 0 || forced == 5) && !pair_off && N % WgradPers::BN == 0 && M >= 128) {
+    GemmParams both = p;
+    both.N = 2 * N;
+    both.split = N;
+    both.out2 = static_cast<uint16_t*>(out1);
+    const int rc = launch_wgrad_persistent(both, num_banks, stream);
+    if (rc <= 0) return rc;
   }
-  if (cfg == 5) cfg = 3;
-  switch (cfg) {
-    case 3: return launch_wgrad<CfgSquare>(p, num_banks, stream);
-    case 1: return launch_wgrad<CfgWide>(p, num_banks, stream);
-    default: return launch_wgrad<CfgSmall>(p, num_banks, stream);
-  }
+  const int rc = launch_tn(p, num_banks, stream);
+  if (rc != NESTOR_HIP_OK) return rc;
+  p.b0 = static_cast<const uint16_t*>(g) + N;
+  p.out = static_cast<uint16_t*>(out1);
+  return launch_tn(p, num_banks, stream);
 }
 
 #if NESTOR_GEMM_CLOCK_HOOK

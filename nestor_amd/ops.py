@@ -608,6 +608,37 @@ def _(a, g, offs, seg_start, seg_count, out_f32=False):
                        dtype=torch.float32 if out_f32 else torch.bfloat16)
 
 
+@torch.library.custom_op(f"{_NS}::grouped_gemm_tn_pair", mutates_args=(), device_types="cuda")
+def grouped_gemm_tn_pair(
+    a: Tensor, g: Tensor, offs: Tensor, seg_start: Tensor | None, seg_count: Tensor | None,
+    out_f32: bool = False,
+) -> list[Tensor]:
+    """``[a_seg^T @ g_seg[:, :N], a_seg^T @ g_seg[:, N:]]`` for ``g [rows_pad, 2N]``: the
+    weight gradients of the fused up|gate GEMM, one launch when ``N % 256 == 0``."""
+
+    assert a.dtype == torch.bfloat16 and g.dtype == torch.bfloat16
+    assert a.stride(1) == 1 and g.stride(1) == 1 and g.shape[1] % 2 == 0
+    rows_pad, m = a.shape
+    n = g.shape[1] // 2
+    num_banks = offs.shape[0]
+    out_dtype = torch.float32 if out_f32 else torch.bfloat16
+    out0 = torch.empty(num_banks, m, n, dtype=out_dtype, device=a.device)
+    out1 = torch.empty(num_banks, m, n, dtype=out_dtype, device=a.device)
+    _lib.call(
+        "nestor_hip_grouped_gemm_tn_pair", _ptr(a), a.stride(0), _ptr(g), g.stride(0), _ptr(out0),
+        _ptr(out1), n, m * n, rows_pad, m, n, num_banks, _ptr(offs.contiguous()), _ptr(seg_start),
+        _ptr(seg_count), _code(out_dtype), _stream(a),
+    )
+    return [out0, out1]
+
+
+@grouped_gemm_tn_pair.register_fake
+def _(a, g, offs, seg_start, seg_count, out_f32=False):
+    dtype = torch.float32 if out_f32 else torch.bfloat16
+    shape = (offs.shape[0], a.shape[1], g.shape[1] // 2)
+    return [a.new_empty(shape, dtype=dtype), a.new_empty(shape, dtype=dtype)]
+
+
 @torch.library.custom_op(f"{_NS}::upgate_swiglu_fwd", mutates_args=(), device_types="cuda")
 def upgate_swiglu_fwd(
     x_pad: Tensor, w_up: Tensor, w_gate: Tensor, tile_table: Tensor
@@ -840,9 +871,11 @@ def _upgate_backward(ctx, grads):
     gx = gup = ggate = None
     if ctx.needs_input_grad[0]:
         gx = grouped_gemm_nt_upgate(g, w_up, w_gate, tile_table)
-    if ctx.needs_input_grad[1]:
+    if ctx.needs_input_grad[1] and ctx.needs_input_grad[2]:
+        gup, ggate = grouped_gemm_tn_pair(x_pad, g, offs, seg_start, seg_count)
+    elif ctx.needs_input_grad[1]:
         gup = grouped_gemm_tn(x_pad, g[:, :h], offs, seg_start, seg_count)
-    if ctx.needs_input_grad[2]:
+    elif ctx.needs_input_grad[2]:
         ggate = grouped_gemm_tn(x_pad, g[:, h:], offs, seg_start, seg_count)
     return gx, gup, ggate, None, None, None, None
 
@@ -881,9 +914,11 @@ def _upgate_owned_backward(ctx, grads):
     gx = gown_up = gown_gate = None
     if ctx.needs_input_grad[0]:
         gx = grouped_gemm_nt_upgate(g, w_up, w_gate, tile_table)
-    if ctx.needs_input_grad[3]:
+    if ctx.needs_input_grad[3] and ctx.needs_input_grad[4]:
+        gown_up, gown_gate = grouped_gemm_tn_pair(x_pad, g, offs, seg_start, seg_count, True)
+    elif ctx.needs_input_grad[3]:
         gown_up = grouped_gemm_tn(x_pad, g[:, :h], offs, seg_start, seg_count, True)
-    if ctx.needs_input_grad[4]:
+    elif ctx.needs_input_grad[4]:
         gown_gate = grouped_gemm_tn(x_pad, g[:, h:], offs, seg_start, seg_count, True)
     return gx, None, None, gown_up, gown_gate, None, None, None, None
 
@@ -1500,7 +1535,7 @@ def register_flop_formulas() -> None:
               "grouped_gemm_fp8w_nn"), _flops_rows_bank),
             (("upgate_swiglu", "upgate_swiglu_owned", "upgate_swiglu_fwd", "grouped_gemm_nt_upgate",
               "grouped_gemm_fp8w_upgate_swiglu"), _flops_upgate),
-            (("grouped_gemm_tn",), _flops_weight_grad),
+            (("grouped_gemm_tn", "grouped_gemm_tn_pair"), _flops_weight_grad),
             (("score_heads",), _flops_score_heads),
         ):
             for name in names:

@@ -23,7 +23,7 @@ _P, _I32, _I64 = c_void_p, c_int32, c_int64
 GEMM_ENTRY_POINTS = (
     "nestor_hip_grouped_gemm_nn", "nestor_hip_grouped_gemm_upgate_swiglu",
     "nestor_hip_grouped_gemm_nt", "nestor_hip_grouped_gemm_nt_upgate",
-    "nestor_hip_grouped_gemm_tn",
+    "nestor_hip_grouped_gemm_tn", "nestor_hip_grouped_gemm_tn_pair",
 )
 _SIGNATURES: dict[str, list] = {
     "nestor_hip_dma_stream_probe": [_P, _I64, _I64, _I64, _I32, _I32, _P],
@@ -63,7 +63,7 @@ def wall_clock_khz() -> int:
 
 @contextlib.contextmanager
 def instrumented(sink_ptr: int):
-    """Inside the block the package's five bf16 grouped-GEMM calls run the measurement
+    """Inside the block the package's bf16 grouped-GEMM calls run the measurement
     library's instrumented build, which adds each workgroup's {shader cycles, wall ticks,
     1, K steps} to the 64 x 4 uint64 device array at ``sink_ptr`` (zeroed by the caller).
     Synchronise the device before entering and before leaving."""

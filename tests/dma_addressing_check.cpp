@@ -91,8 +91,27 @@ void check_rows(int64_t K, int64_t N, int64_t lda, int64_t ldb, int nrows, int64
 }
 
 // The persistent weight gradient's descriptors over one segment and one tile.
+template <int TILE>
 void check_wgrad(int64_t rows_total, int64_t beg, int seg_rows, int64_t ld, int64_t cols, int m0) {
-  constexpr int BK = 32, TILE = 256, WAVES = 4, CHUNKS = 4;
+  constexpr int BK = 32, WAVES = 4, CHUNKS = TILE * BK / 8 / (64 * WAVES);
+  if (ld >= TILE) {  // (a narrower row does not tell a piece's row from its byte offset)
+    // a K step's transfers fetch every 16-byte piece of its BK rows x TILE columns exactly once
+    std::vector<int> seen(BK * (TILE / 8), 0);
+    for (int wave = 0; wave < WAVES; ++wave)
+      for (int c = 0; c < CHUNKS; ++c)
+        for (int lane = 0; lane < 64; ++lane) {
+          const uint32_t off = wgrad_lane_offset(wave, WAVES, c, lane, ld, TILE);
+          const int64_t krow = off / (ld * 2), piece = off % (ld * 2) / 16;
+          REQUIRE(krow < BK && piece < TILE / 8, "wgrad piece (%ld, %ld) outside the K step", (long)krow, (long)piece);
+          // where the transfer puts it: lanes fill the instruction's KiB in order, which must be
+          // the swizzled slot that the transposing reads expect
+          const int slot = ((wave + WAVES * c) * 64 + lane);
+          const int want = static_cast<int>(krow) * (TILE / 8) + (static_cast<int>(piece) ^ (4 * (static_cast<int>(krow) & 3)));
+          REQUIRE(slot == want, "wgrad piece (%ld, %ld) lands in slot %d, read from %d", (long)krow, (long)piece, slot, want);
+          ++seen[krow * (TILE / 8) + piece];
+        }
+    for (size_t i = 0; i < seen.size(); ++i) REQUIRE(seen[i] == 1, "wgrad piece %zu fetched %d times", i, seen[i]);
+  }
   const int64_t operand_bytes = rows_total * ld * 2;
   int64_t base = (beg * ld + m0) * 2;  // bytes from the operand's start
   int64_t records = wgrad_num_records(seg_rows, ld, cols, m0, TILE);
@@ -106,7 +125,7 @@ void check_wgrad(int64_t rows_total, int64_t beg, int seg_rows, int64_t ld, int6
     for (int wave = 0; wave < WAVES; ++wave)
       for (int c = 0; c < CHUNKS; ++c)
         for (int lane = 0; lane < 64; ++lane) {
-          const uint32_t off = wgrad_lane_offset(wave, WAVES, c, lane, ld);
+          const uint32_t off = wgrad_lane_offset(wave, WAVES, c, lane, ld, TILE);
           // the hardware drops what lies at or behind num_records; what it lets through
           // must be rows of this segment
           if (static_cast<int64_t>(off) + 16 <= records) {
@@ -163,11 +182,18 @@ int main() {
   for (int seg_rows : {1, 2, 16, 31, 32, 33, 100, 512, 530})
     for (int64_t cols : {64, 160, 216, 256, 264, 424, 2048})
       for (int64_t ld : {cols, cols + 8, 2 * cols})
+      {
         for (int m0 = 0; m0 < cols; m0 += 256) {
-          check_wgrad(seg_rows, 0, seg_rows, ld, cols, m0);                 // the operand is this segment
-          check_wgrad(600 + seg_rows, 600, seg_rows, ld, cols, m0);         // the last segment of a longer operand
-          check_wgrad(2000, 48, seg_rows, ld, cols, m0);
+          check_wgrad<256>(seg_rows, 0, seg_rows, ld, cols, m0);            // the operand is this segment
+          check_wgrad<256>(600 + seg_rows, 600, seg_rows, ld, cols, m0);    // the last segment of a longer operand
+          check_wgrad<256>(2000, 48, seg_rows, ld, cols, m0);
         }
+        for (int m0 = 0; m0 < cols; m0 += 128) {                            // the 128-column tile
+          check_wgrad<128>(seg_rows, 0, seg_rows, ld, cols, m0);
+          check_wgrad<128>(600 + seg_rows, 600, seg_rows, ld, cols, m0);
+          check_wgrad<128>(2000, 48, seg_rows, ld, cols, m0);
+        }
+      }
   std::printf("ok: %ld checks\n", checks);
   return 0;
 }

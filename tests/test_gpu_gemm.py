@@ -128,6 +128,38 @@ def test_upgate_swiglu_fused_matches_unfused(cuda, tokens, slots, banks, K, H, s
     assert rel_l2(tg.grad, gf.grad) < 1e-2
 
 
+@pytest.mark.parametrize("tokens,slots,banks,K,H,skew", [
+    (2048, 2, 8, 1024, 512, False),   # one launch: column tiles never straddle the halves
+    (1200, 2, 24, 264, 256, True),    # one launch, overhanging row tiles, empty banks
+    (900, 3, 5, 640, 216, True),      # widths that fall back to two launches
+    (300, 2, 6, 40, 24, False),
+])
+@pytest.mark.parametrize("out_f32", [False, True])
+def test_weight_gradient_pair_equals_two_calls(cuda, tokens, slots, banks, K, H, skew, out_f32):
+    """Both weight gradients of the fused up|gate GEMM in one call: the same bits as one
+    call per half, and both against an fp32 per-segment product."""
+
+    from nestor_amd import ops
+
+    want, got = _setup(tokens, slots, banks, cuda, skew)
+    a = _padded_input(want, K, 11)
+    g = _padded_input(want, 2 * H, 12)
+    ta, tg = a.to(cuda), g.to(cuda)
+    for starts, counts in ((None, None), (got.padded_starts, got.kept_counts)):
+        pair = ops.grouped_gemm_tn_pair(ta, tg, got.offs, starts, counts, out_f32)
+        one = [ops.grouped_gemm_tn(ta, tg[:, :H], got.offs, starts, counts, out_f32),
+               ops.grouped_gemm_tn(ta, tg[:, H:], got.offs, starts, counts, out_f32)]
+        for half in range(2):
+            assert pair[half].dtype == (torch.float32 if out_f32 else torch.bfloat16)
+            assert torch.equal(pair[half], one[half])
+    bounds = [0] + want.offs.tolist()
+    for half in range(2):
+        ref = torch.stack([a[bounds[i]:bounds[i + 1]].float().t()
+                           @ g[bounds[i]:bounds[i + 1], half * H:(half + 1) * H].float()
+                           for i in range(banks)])
+        assert rel_l2(pair[half], ref) < 4e-3
+
+
 def test_slack_tail_is_zero_filled(cuda):
     """Rows behind the last segment belong to no bank: outputs there are zeros
     even when the output buffer held garbage."""

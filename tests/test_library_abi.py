@@ -41,7 +41,7 @@ def test_measurement_aids_live_in_their_own_library():
     # the instrumented GEMM entry points carry the product's names and signatures
     for name in ("nestor_hip_grouped_gemm_nn", "nestor_hip_grouped_gemm_upgate_swiglu",
                  "nestor_hip_grouped_gemm_nt", "nestor_hip_grouped_gemm_nt_upgate",
-                 "nestor_hip_grouped_gemm_tn"):
+                 "nestor_hip_grouped_gemm_tn", "nestor_hip_grouped_gemm_tn_pair"):
         assert hasattr(plib, name)
     lib = ctypes.CDLL(str(_lib.LIB_PATH))
     for name in probes:
