@@ -167,6 +167,13 @@ int main() {
         check_rows<128, 256, 64, 4, true, 1>(1280, N, 1280, 1280, nrows, n0, 1);
         check_rows<128, 256, 64, 4, false, 1>(1280, N, 1280, N, nrows, n0, 1);
       }
+  // input gradients narrower than a column tile (h = 136 .. 248): rows of the weight tile
+  // behind the last output column are re-reads of that column
+  for (int nrows : {1, 100, 320})
+    for (int64_t N : {136, 160, 216, 248}) {
+      check_rows<320, 256, 32, 4, true, 1>(1280, N, 1280, 1280, nrows, 0, 1);
+      check_rows<320, 256, 32, 4, true, 1>(424, N, 848, 424, nrows, 0, 2);   // fused, narrow model width
+    }
   // contractions that end inside a K step (the production widths 424, 216, 184; the shortest ones)
   for (int64_t K : {8, 24, 40, 184, 216, 424})
     for (int nrows : {1, 100, 160}) {

@@ -50,6 +50,9 @@ SHAPES = [
     (900, 3, 5, 216, 640, False),
     (640, 1, 3, 8, 512, False),
     (1100, 2, 4, 640, 184, False),
+    # input gradients narrower than the 256-column tile (h = 160 / 136 of the production arms)
+    (1500, 2, 6, 160, 1280, True),
+    (700, 2, 5, 136, 512, False),
 ]
 
 
