@@ -277,6 +277,27 @@ def timed_steps(w, column_router, pool, x, grad_out, steps: int, warmup: int, au
     return ms
 
 
+def graphed_steps(w, column_router, pool, x, grad_out, steps: int) -> float:
+    """ms per step of the same pass replayed as one HIP graph (``GraphedStep``): what the
+    step costs once the host's ~150 launches per step are out of the way."""
+
+    from nestor_amd.workloads import GraphedStep
+
+    params = list(column_router.parameters()) + list(pool.parameters())
+    graphed = GraphedStep(w, column_router, pool, x, grad_out)
+    graphed()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graphed()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    del graphed
+    for p in params:
+        p.grad = None
+    return ms
+
+
 def extra_shapes(dev, seed: int) -> dict:
     """The path at the reference's production widths (registered ``nestor_*`` arms: d that
     is no power of two, private widths of 160-424, 6-16 slots per token, 120 private
@@ -292,6 +313,7 @@ def extra_shapes(dev, seed: int) -> dict:
         column_router, pool = build_pool(w, t)
         x = t.x.clone().requires_grad_(True)
         ms = timed_steps(w, column_router, pool, x, t.grad_out, 5, 2, False)
+        ms_graph = graphed_steps(w, column_router, pool, x, t.grad_out, 10)
         flops = w.gemm_flops()
         routed = routed_slots(w, t, column_router, pool)
         entry = {
@@ -299,7 +321,9 @@ def extra_shapes(dev, seed: int) -> dict:
                      f"top-{w.k_columns} columns x top-{w.k_private} = {w.k_columns * w.k_private} slots; "
                      f"public {w.public} h={w.h_public} top-{w.k_public}",
             "ms_per_step": round(ms, 3),
+            "ms_per_step_hip_graph": round(ms_graph, 3),
             "tokens_per_s": round(w.tokens / ms * 1e3, 1),
+            "tokens_per_s_hip_graph": round(w.tokens / ms_graph * 1e3, 1),
             "expert_gemm_tflops": round(flops / ms / 1e9, 1),
             "expert_gemm_frac_mfma_peak": round(flops / ms / 1e9 / BF16_MFMA_PEAK_TFLOPS, 4),
         }

@@ -159,3 +159,61 @@ def expert_mlp_step(w: Workload, column_router, pool, x: Tensor, grad_out: Tenso
     if grad_out is not None:
         update.backward(grad_out.view_as(update))
     return update
+
+
+class GraphedStep:
+    """``expert_mlp_step`` (forward + backward) captured into one HIP graph and replayed.
+
+    Nothing about the path's launches depends on the routing (static grids, device-side tile
+    tables, no host read-backs), so a step is ~150 launches with fixed arguments: at the
+    production widths the host spends longer issuing them than the device takes to run them,
+    and a replay removes that cost.  ``x`` and ``grad_out`` are copied into buffers the graph
+    owns; the update, ``x_grad`` and every parameter's ``.grad`` are graph-owned tensors that
+    each replay overwrites (gradients are assigned, not accumulated: they are ``None`` when
+    the capture starts)."""
+
+    def __init__(self, w: Workload, column_router, pool, x: Tensor, grad_out: Tensor,
+                 autocast: bool = False, warmup: int = 3) -> None:
+        self.params = list(column_router.parameters()) + list(pool.parameters())
+        self.x = x.detach().clone().requires_grad_(True)
+        self.grad_out = grad_out.detach().clone()
+        dev = x.device
+
+        def step():
+            with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+                return expert_mlp_step(w, column_router, pool, self.x, self.grad_out)
+
+        def drop_grads():
+            for p in self.params:
+                p.grad = None
+            self.x.grad = None
+
+        import warnings
+
+        main = torch.cuda.current_stream(dev)
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(main)
+        with warnings.catch_warnings():
+            # the parameters were made on another stream than the capture's: autograd says so
+            # once; the replays are checked against eager steps bit for bit in the tests
+            warnings.filterwarnings("ignore", message=".*AccumulateGrad node's stream.*")
+            with torch.cuda.stream(side):
+                for _ in range(warmup):
+                    drop_grads()
+                    step()
+            main.wait_stream(side)
+            torch.cuda.synchronize(dev)
+            drop_grads()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.update = step()
+        self.x_grad = self.x.grad
+
+    def __call__(self, x: Tensor | None = None, grad_out: Tensor | None = None) -> Tensor:
+        if x is not None:
+            self.x.detach().copy_(x)
+        if grad_out is not None:
+            self.grad_out.copy_(grad_out)
+        self.graph.replay()
+        return self.update
+

@@ -371,3 +371,50 @@ def test_config_fp8_inference_bank(cuda, tokens):
         assert err < 3e-2
         del q, deq, gold
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("workload", ["tiny_100m", "nestor_200m_block0"])
+def test_graphed_step_replays_equal_eager_steps(cuda, workload):
+    """The whole forward + backward step captured into one HIP graph: every replay -- on new
+    inputs, with eager work and synchronisations between the replays -- gives the bits of the
+    eager step on the same inputs (update, input gradient and every parameter gradient)."""
+
+    from nestor_amd.workloads import WORKLOADS, GraphedStep, build_pool, expert_mlp_step, make_tensors
+
+    w = WORKLOADS[workload]
+    t = make_tensors(w, 0, cuda)
+    column_router, pool = build_pool(w, t)
+    params = list(column_router.parameters()) + list(pool.parameters())
+
+    def eager(x, grad_out):
+        for p in params:
+            p.grad = None
+        xe = x.clone().requires_grad_(True)
+        update = expert_mlp_step(w, column_router, pool, xe, grad_out)
+        torch.cuda.synchronize()
+        grads = [None if p.grad is None else p.grad.clone() for p in params]
+        return update.detach().clone(), xe.grad.clone(), grads
+
+    graphed = GraphedStep(w, column_router, pool, t.x, t.grad_out)
+    graph_grads = [p.grad for p in params]   # graph-owned, overwritten by each replay
+    g = torch.Generator(device=cuda).manual_seed(5)
+    for replay in range(4):
+        scale = 1.0 + 0.25 * replay
+        x = (t.x * scale + 0.01 * torch.randn(t.x.shape, generator=g, device=cuda, dtype=torch.float32).to(t.x.dtype))
+        grad_out = t.grad_out * (1.0 - 0.1 * replay)
+        update = graphed(x, grad_out).detach().clone()
+        torch.cuda.synchronize()
+        got_x = graphed.x_grad.clone()
+        got = [None if gg is None else gg.clone() for gg in graph_grads]
+        # the eager step runs between the replays (its own launches, allocations, a sync)
+        for p, gg in zip(params, graph_grads):
+            p.grad = None
+        want_update, want_x, want = eager(x, grad_out)
+        for p, gg in zip(params, graph_grads):
+            p.grad = gg
+        assert torch.equal(update, want_update), (workload, replay, "update")
+        assert torch.equal(got_x, want_x), (workload, replay, "x.grad")
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert (a is None) == (b is None), (workload, replay, i)
+            if a is not None:
+                assert torch.equal(a, b), (workload, replay, f"parameter {i}")
