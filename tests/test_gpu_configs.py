@@ -135,13 +135,14 @@ def _gold_step(w, t, column_router, pool, priv_ids, pub_ids):
 
 
 def _record_rel_l2(workload: str, seed: int, errors: dict) -> None:
-    """Appends the measured figures to ``gpurun_out/parity_rel_l2.md`` (one table row per
-    tensor) when that folder exists: the record behind the tolerances quoted for this
-    path.  The tracked copy is ``profiles/parity_rel_l2.md``."""
+    """Appends the measured figures to ``parity_rel_l2.md`` (one table row per tensor) in the
+    run's scratch output folder, when there is one: the record behind the tolerances quoted
+    for this path.  The tracked copy is ``profiles/parity_rel_l2.md``."""
 
     import os
 
-    folder = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    folder = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                          os.environ.get("NESTOR_TEST_OUTPUT_DIR", "gpurun_out"))
     if not os.path.isdir(folder):
         return
     path = os.path.join(folder, "parity_rel_l2.md")
