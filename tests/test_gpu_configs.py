@@ -217,11 +217,11 @@ def test_config_step_outputs_and_all_gradients_vs_fp32(cuda, workload, seeds):
         torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("workload", ["nestor_1b_block0", "nestor_200m_block0"])
+@pytest.mark.parametrize("workload", ["nestor_1b_block0", "nestor_1b_block6", "nestor_200m_block0"])
 def test_production_widths_bank_calls_vs_fp32(cuda, workload):
     """The reference's registered arms at their real widths (d = 1280 / 640, private experts
-    424 / 216 wide, 6 slots per token over 120 / 64 private experts, 8 public experts top-2
-    of width d): both bank calls of a whole micro-batch, forward and backward, on the ids
+    424 / 160 / 216 wide, 6 / 16 / 6 slots per token over 120 / 120 / 64 private experts, 8
+    public experts top-2 of width d): both bank calls of a whole micro-batch, forward and backward, on the ids
     the routers produced, against the fp32 gold -- outputs, input and slot-weight gradients
     and all six bank gradients within 1e-2."""
 
