@@ -383,7 +383,7 @@ def mfma_clock_probe(dev, iters: int = 100000) -> dict:
     return out
 
 
-def traffic_probe(w, tensors, routed) -> None:
+def traffic_probe(w, tensors, routed, uniform: bool = False) -> None:
     """Yardsticks of known size for the HBM counters, then the private bank's up|gate
     kernel on the workload's routing.  Run under `rocprofv3 --pmc FETCH_SIZE` and again
     under `--pmc WRITE_SIZE`; each launch below is one dispatch in the counter output:
@@ -395,7 +395,11 @@ def traffic_probe(w, tensors, routed) -> None:
     2. torch's elementwise copy of the 128 MiB activations (reads and writes 128 MiB);
     3. ``dispatch_fwd_kernel`` (16-byte lanes, 4 KiB rows: the store shape of the GEMM
        epilogues) writing ``rows_pad * d * 2`` bytes;
-    4. ``grouped_gemm_dma_kernel<..., kNNUpGate>`` twice."""
+    4. ``grouped_gemm_dma_kernel<..., kNNUpGate>`` twice.
+
+    ``uniform``: every bank gets the same number of rows (ids in round-robin order) instead of
+    the routers' choice: whole 128-row tiles, four per bank, so that a tile order which
+    keeps a bank's row tiles on one XCD is exactly aligned."""
 
     import ctypes
 
@@ -407,6 +411,8 @@ def traffic_probe(w, tensors, routed) -> None:
     slots = w.k_columns * w.k_private
     banks = w.columns * w.private
     ids = routed[0].reshape(-1).contiguous()
+    if uniform:
+        ids = (torch.arange(ids.numel(), device=dev, dtype=ids.dtype) % banks).contiguous()
     plan = dispatch_plan(ids, banks, slots, torch.bfloat16)
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     buf = torch.empty(1 << 30, dtype=torch.bfloat16, device=dev).normal_()   # 2 GiB
@@ -607,6 +613,9 @@ def main() -> None:
                     help="launch yardsticks of known size (LDS-DMA streams, a copy, a row kernel) and "
                          "the dominant kernel twice, then exit: the command to run under "
                          "`rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`")
+    ap.add_argument("--traffic-uniform", action="store_true",
+                    help="with --traffic-probe: the same number of rows for every bank instead of the "
+                         "routers' choice")
     ap.add_argument("--fp8-probe", action="store_true",
                     help="time the e4m3-weight forward at 64/256/1024 tokens and print one JSON "
                          "line (HBM GB/s over the weights of the experts that received a row)")
@@ -632,7 +641,7 @@ def main() -> None:
     with torch.autocast("cuda", dtype=torch.bfloat16, enabled=fp32_owners):
         routed = routed_slots(w, tensors, column_router, pool)
     if args.traffic_probe:
-        traffic_probe(w, tensors, routed)
+        traffic_probe(w, tensors, routed, args.traffic_uniform)
         return
     if args.fp8_probe:
         print(json.dumps({"workload": f"{w.name}, e4m3 weights, forward only",
