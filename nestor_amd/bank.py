@@ -184,12 +184,28 @@ class StackedExpertBank(nn.Module):
 
         self.__dict__.pop("_shadow", None)
 
-    def refresh_shadow(self) -> None:
-        """Rebuild the bf16 copies from the owners now."""
+    def refresh_shadow(self, in_place: bool = False) -> None:
+        """Rebuild the bf16 copies from the owners now.
+
+        ``in_place``: rewrite the existing copies instead of making new tensors, so that
+        their addresses stay what a captured HIP graph of the step reads (the replays do
+        not re-run this host-side check: call this after every optimizer step, outside the
+        graph).  Only between steps: an autograd graph that saved the copies and has not
+        run its backward yet would see them change under it."""
 
         owners = (self.w_up, self.w_gate, self.w_down)
+        cached = self.__dict__.get("_shadow")
         with torch.no_grad():
-            copies = tuple(None if o is None else o.detach().to(torch.bfloat16) for o in owners)
+            if in_place and cached is not None and all(
+                (c is None) == (o is None) and (c is None or (c.shape == o.shape and c.device == o.device))
+                for c, o in zip(cached[1], owners)
+            ):
+                copies = cached[1]
+                for c, o in zip(copies, owners):
+                    if c is not None:
+                        c.copy_(o.detach())
+            else:
+                copies = tuple(None if o is None else o.detach().to(torch.bfloat16) for o in owners)
         key = tuple(None if o is None else (o.data_ptr(), o._version) for o in owners)
         self.__dict__["_shadow"] = (key, copies)
 

@@ -186,6 +186,14 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
                 bank.enable_bf16_shadow(enabled)
         return self
 
+    def refresh_shadow(self, in_place: bool = False) -> None:
+        """``StackedExpertBank.refresh_shadow`` on both stacked banks (after an optimizer step
+        when the step is replayed as a captured graph: ``in_place=True``)."""
+
+        for bank in (self.stacked_public, self.stacked_private):
+            if bank is not None and bank.__dict__.get("_shadow_enabled", False):
+                bank.refresh_shadow(in_place)
+
     # -- slots ---------------------------------------------------------------
     def _private_bank(self) -> list[nn.Module]:
         if self.private_experts is None:

@@ -170,7 +170,9 @@ class GraphedStep:
     and a replay removes that cost.  ``x`` and ``grad_out`` are copied into buffers the graph
     owns; the update, ``x_grad`` and every parameter's ``.grad`` are graph-owned tensors that
     each replay overwrites (gradients are assigned, not accumulated: they are ``None`` when
-    the capture starts)."""
+    the capture starts).  With fp32 owners behind a bf16 shadow the replays read the copies
+    that existed at capture: after every optimizer step call
+    ``pool.refresh_shadow(in_place=True)`` before the next replay."""
 
     def __init__(self, w: Workload, column_router, pool, x: Tensor, grad_out: Tensor,
                  autocast: bool = False, warmup: int = 3) -> None:

@@ -419,3 +419,46 @@ def test_graphed_step_replays_equal_eager_steps(cuda, workload):
             assert (a is None) == (b is None), (workload, replay, i)
             if a is not None:
                 assert torch.equal(a, b), (workload, replay, f"parameter {i}")
+
+
+def test_graphed_step_with_bf16_shadow_follows_an_optimizer_step(cuda):
+    """fp32 owners behind the bf16 shadow under autocast, the step replayed as a HIP graph:
+    after an in-place update of the owners and ``refresh_shadow(in_place=True)`` the replay
+    equals the eager step on the updated owners (the graph reads the rewritten copies)."""
+
+    from nestor_amd.workloads import WORKLOADS, GraphedStep, build_pool, expert_mlp_step, make_tensors
+
+    w = WORKLOADS["tiny_100m"]
+    t = make_tensors(w, 0, cuda, torch.float32)
+    column_router, pool = build_pool(w, t)
+    pool.enable_bf16_shadow()
+    params = list(column_router.parameters()) + list(pool.parameters())
+
+    def eager():
+        for p in params:
+            p.grad = None
+        xe = t.x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            update = expert_mlp_step(w, column_router, pool, xe, t.grad_out)
+        torch.cuda.synchronize()
+        return update.detach().clone(), xe.grad.clone(), pool.stacked_private.w_up.grad.clone()
+
+    graphed = GraphedStep(w, column_router, pool, t.x, t.grad_out, autocast=True)
+    graph_grads = [p.grad for p in params]
+    owner = pool.stacked_private.w_up
+    owner_slot = [i for i, p in enumerate(params) if p is owner][0]
+    for round_ in range(3):
+        update = graphed().detach().clone()
+        torch.cuda.synchronize()
+        got_x, got_w = graphed.x_grad.clone(), graph_grads[owner_slot].clone()
+        want_update, want_x, want_w = eager()
+        for p, gg in zip(params, graph_grads):
+            p.grad = gg
+        assert torch.equal(update, want_update), round_
+        assert torch.equal(got_x, want_x), round_
+        assert got_w.dtype == torch.float32 and torch.equal(got_w, want_w), round_
+        with torch.no_grad():   # an optimizer step on every bank tensor
+            for bank in (pool.stacked_public, pool.stacked_private):
+                for name in ("w_up", "w_gate", "w_down"):
+                    getattr(bank, name).mul_(1.0 - 0.05 * (round_ + 1))
+        pool.refresh_shadow(in_place=True)

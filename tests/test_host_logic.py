@@ -224,6 +224,14 @@ def test_bf16_shadow_follows_data_writes():
     bank.w_gate.data.copy_(w3[1] * 5)
     bank.refresh_shadow()
     assert torch.equal(copies()[1], (w3[1] * 5).bfloat16())
+    # in place: the copies keep their storage (what a captured graph of the step reads)
+    before = [c.data_ptr() for c in copies()]
+    with torch.no_grad():
+        bank.w_up.add_(1.0)
+    bank.refresh_shadow(in_place=True)
+    after = copies()
+    assert [c.data_ptr() for c in after] == before
+    assert torch.equal(after[0], bank.w_up.detach().bfloat16())
     # loading a state dict drops the copy
     state = {k: v.clone() * 0.5 for k, v in bank.state_dict().items()}
     bank.load_state_dict(state)
