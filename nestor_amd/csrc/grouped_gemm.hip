@@ -1466,9 +1466,13 @@ int launch_rows_dma(GemmParams p, int table_kind, int64_t rows_pad, int32_t num_
 #endif
   static const int forced_group = config_choice("NESTOR_HIP_TILE_GROUP", -1);
   // Measured at the 1b-like shapes: the down projection runs best (and fetches least)
-  // with eight row tiles per XCD group walked row tile first; the fused input gradient
-  // with four, column tile first; the others in plain order.  The spread is 2-6 %.
-  p.tile_group = forced_group >= 0 ? forced_group : (kMode == kNN ? 8 : kMode == kNTUpGate ? 4 : 0);
+  // with a bank's row tiles per XCD group walked row tile first (four tiles for banks of
+  // ~512 rows: 1.33 -> 1.27 ms against groups of eight; eight for banks of thousands of
+  // rows); the fused input gradient with four, column tile first; the others in plain
+  // order.  The spread is 2-6 %.
+  const int64_t tiles_per_bank = rows_pad / num_banks / 128;
+  p.tile_group = forced_group >= 0 ? forced_group
+                                   : (kMode == kNN ? (tiles_per_bank <= 5 ? 4 : 8) : kMode == kNTUpGate ? 4 : 0);
   static const int forced_order = config_choice("NESTOR_HIP_TILE_ORDER", -1);
   p.tile_order = forced_order >= 0 ? forced_order : (kMode == kNN ? 1 : 0);
   // whole groups of row tiles per XCD (see the kernel's tile mapping)
