@@ -23,7 +23,7 @@ from nestor_amd import flags, ops
 from nestor_amd.bank import Linear2, StackedBanksMixin, SwigluExpert
 from nestor_amd.grouped import grouped_expert_combine
 from nestor_amd.router import (
-    Router, RouterOutput, _refuse_noise, check_batchable, route_private_batched, score_linear,
+    Router, RouterOutput, check_batchable, route_private_batched, score_linear,
 )
 
 
@@ -71,11 +71,6 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
         super().__init__()
         if num_private_experts < 1:
             raise ValueError("ExpertPoolMLP requires a private pool: num_private_experts must be > 0.")
-        if router_noise_mlp_hidden_dims is not None:
-            raise NotImplementedError(
-                "router exploration noise (router_noise_mlp_hidden_dims) is not part of this "
-                "implementation; construct the pool without it"
-            )
         if not 1 <= num_groups_per_token <= num_groups:
             raise ValueError("num_groups_per_token must be in [1, num_groups].")
         self.dim = dim
@@ -98,7 +93,8 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
 
         def make_router(choices: int, top_k: int, gate_mode: str = "renorm") -> Router:
             return Router(dim, choices, top_k, router_score_mlp_hidden_dims,
-                          router_score_mlp_activation, loss_free_balancing=loss_free_balancing,
+                          router_score_mlp_activation, router_noise_mlp_hidden_dims,
+                          router_noise_mlp_activation, loss_free_balancing=loss_free_balancing,
                           bias_update_rate=bias_update_rate, gate_mode=gate_mode)
 
         self.public_router = make_router(num_public_experts, public_top_k) if self.has_public_pool else None
@@ -270,30 +266,60 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
         return (out[:, :n_pub].reshape(*x.shape[:-1], n_pub), out[:, n_pub:n_pub + n_priv],
                 out[:, n_pub + n_priv:].reshape(*x.shape[:-1], -1))
 
-    def _route(self, x: Tensor, valid: Tensor, group_active: Tensor):
+    def _route(self, x: Tensor, valid: Tensor, group_active: Tensor, router_noise=None):
         """``(public_output, private_outputs, stacked, path_logits)``: ``stacked`` holds the
         batched routers' ``[B, S, G, Q]`` gates and ``[B, S, G, k]`` choices (``None`` for
         per-column routers), ``path_logits`` the path gate's scores when the fused score
-        GEMM produced them (``None``: the caller evaluates the path gate itself)."""
+        GEMM produced them (``None``: the caller evaluates the path gate itself).
 
+        The public router runs first, then the ``G`` private ones: routers with a noise
+        head draw from the RNG in training mode, so the order is part of the contract
+        (nestor/backbones/expert_pools.py:533-586).  ``router_noise``: the pre-drawn
+        factors of ``draw_router_noise`` (``"public"`` ``[B, S, P]``, ``"private"``
+        ``[B, S, G, Q]``); ``None`` lets each router draw its own."""
+
+        public_noise = None if router_noise is None else router_noise.get("public")
+        private_noise = None if router_noise is None else router_noise.get("private")
         fused = self._fused_head_scores(x)
         if fused is not None:
             pub_scores, priv_scores, path_logits = fused
-            public_output = self.public_router(x, valid, scores=pub_scores)
+            public_output = self.public_router(x, valid, noise=public_noise, scores=pub_scores)
             outs, gates, choices = route_private_batched(
                 list(self.private_routers), x, valid, group_active, training=self.training,
-                scores=priv_scores,
+                noise=private_noise, scores=priv_scores,
             )
             return public_output, outs, (gates, choices), path_logits
-        public_output = self.public_router(x, valid) if self.public_router is not None else None
+        public_output = (
+            self.public_router(x, valid, noise=public_noise) if self.public_router is not None else None
+        )
         if self.batched_routers:
             outs, gates, choices = route_private_batched(
-                list(self.private_routers), x, valid, group_active, training=self.training
+                list(self.private_routers), x, valid, group_active, training=self.training,
+                noise=private_noise,
             )
             return public_output, outs, (gates, choices), None
-        outs = [self.private_routers[g](x, valid & group_active[:, :, g])
-                for g in range(self.num_groups)]
+        outs = [
+            self.private_routers[g](
+                x, valid & group_active[:, :, g],
+                noise=None if private_noise is None else private_noise[:, :, g],
+            )
+            for g in range(self.num_groups)
+        ]
         return public_output, outs, None, None
+
+    def draw_router_noise(self, batch_size: int, seq_len: int, device, dtype: torch.dtype) -> dict:
+        """Every pool router's standard-normal noise factor, drawn in one place (outside an
+        activation checkpoint) and handed back through ``router_noise`` so that a recompute
+        routes as the forward did (nestor/backbones/expert_pools.py:588-623): ``"private"``
+        ``[B, S, G, Q]`` and, with a public pool, ``"public"`` ``[B, S, P]``."""
+
+        noise = {
+            "private": torch.randn(batch_size, seq_len, self.num_groups, self.num_private_experts,
+                                   device=device, dtype=dtype)
+        }
+        if self.public_router is not None:
+            noise["public"] = self.public_router.draw_noise(batch_size, seq_len, device, dtype)
+        return noise
 
     # -- banks ---------------------------------------------------------------
     def _bank(self, flat_x: Tensor, experts, stacked, ids: Tensor, weights: Tensor, group: int) -> Tensor:
@@ -317,11 +343,13 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
             logits = self.path_gate(x)
         return F.softmax(logits.float(), dim=-1).to(x.dtype)
 
-    def _prologue(self, x: Tensor, valid: Tensor, group_gates: Tensor, group_active: Tensor):
+    def _prologue(self, x: Tensor, valid: Tensor, group_gates: Tensor, group_active: Tensor,
+                  router_noise=None):
         flat_x = x.reshape(-1, self.dim)
         num_tokens = flat_x.shape[0]
         flat_gates = group_gates.reshape(num_tokens, self.num_groups)
-        public_output, private_outputs, stacked, path_logits = self._route(x, valid, group_active)
+        public_output, private_outputs, stacked, path_logits = self._route(
+            x, valid, group_active, router_noise)
         public_update = (
             self._public_update(flat_x, public_output, num_tokens).reshape_as(x)
             if public_output is not None else None
@@ -334,9 +362,8 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
                 group_active_mask: Tensor, router_noise=None):
         """Summed layout: ``(update [B,S,d], public_output, private_outputs)``."""
 
-        _refuse_noise(router_noise)
         flat_x, n, flat_gates, pub_out, priv_outs, stacked, public_update, path_logits = self._prologue(
-            x, valid_token_mask, group_gates, group_active_mask
+            x, valid_token_mask, group_gates, group_active_mask, router_noise
         )
         ids, weights, _ = self._private_slots(priv_outs, flat_gates, n, stacked=stacked)
         private_update = self._bank(
@@ -355,9 +382,8 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
                          group_active_mask: Tensor, slot_groups: Tensor, router_noise=None):
         """Slot layout: ``(public [B,S,d] | None, private [B,S,k_a,d], ...)``."""
 
-        _refuse_noise(router_noise)
         flat_x, n, flat_gates, pub_out, priv_outs, stacked, public_update, path_logits = self._prologue(
-            x, valid_token_mask, group_gates, group_active_mask
+            x, valid_token_mask, group_gates, group_active_mask, router_noise
         )
         ids, weights, _ = self._private_slots(
             priv_outs, flat_gates, n, selected=slot_groups.reshape(n, self.num_groups_per_token), stacked=stacked
@@ -371,9 +397,8 @@ class ExpertPoolMLP(StackedBanksMixin, nn.Module):
                           group_active_mask: Tensor, router_noise=None):
         """Column layout: ``(public [B,S,d] | None, private [B,S,G,d], ...)``."""
 
-        _refuse_noise(router_noise)
         flat_x, n, flat_gates, pub_out, priv_outs, stacked, public_update, path_logits = self._prologue(
-            x, valid_token_mask, group_gates, group_active_mask
+            x, valid_token_mask, group_gates, group_active_mask, router_noise
         )
         ids, weights, selected = self._private_slots(priv_outs, flat_gates, n, stacked=stacked)
         per_slot = self._private_per_slot(flat_x, ids, weights)

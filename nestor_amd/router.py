@@ -1,14 +1,17 @@
 """Token-choice top-k routers of the expert pools.
 
-Mirrors ``RouterOutput`` / ``Router`` (nestor/backbones/nestor.py:320-593, the
-deterministic forward: score head, softmax, detached choice bias, top-k,
+Mirrors ``RouterOutput`` / ``Router`` (nestor/backbones/nestor.py:320-593: score
+head, training-mode exploration noise, softmax, detached choice bias, top-k,
 ``renorm`` / ``switch`` gate, scatter, validity mask) and the batched evaluation
 of a layer's ``G`` private routers (nestor/backbones/batched_router.py:97-240).
 Everything after the score GEMM -- softmax, biased top-k, gates -- is one HIP
 launch for the whole ``[tokens, (G,) choices]`` block, and the gradient of the
 scores is one more.  The loss-free balancing update of ``choice_bias``
 (nestor/backbones/nestor.py:596-634) takes its counts from a histogram launch.
-Exploration noise belongs to the training loop and is not part of this path.
+A router built with a noise head perturbs its scores in training mode
+(``scores + eps * softplus(noise_mlp(x))``, nestor/backbones/nestor.py:540-556), with
+``eps`` drawn there or handed in pre-drawn so that a checkpoint's recompute routes
+as the forward did; a router built without one is deterministic in both modes.
 
 ``torch.topk`` leaves the order of equal scores open; this implementation (and
 its oracle) take equal biased scores lowest index first.
@@ -118,12 +121,17 @@ def route_scores(
             gates.view(shape))
 
 
-def _refuse_noise(noise) -> None:
-    if noise is not None:
-        raise NotImplementedError(
-            "router exploration noise is not part of this implementation: the deterministic "
-            "forward is the only one built (pass noise=None)"
-        )
+def _is_recomputing() -> bool:
+    """True inside a backward pass, i.e. when an activation checkpoint re-runs a forward
+    (nestor/backbones/nestor.py:1077-1089): per-step counters must not advance then."""
+
+    return torch._C._current_autograd_node() is not None
+
+
+def _anneal_steps_from_env() -> int:
+    import os
+
+    return int(os.environ.get("NESTOR_ROUTER_NOISE_ANNEAL_STEPS", "0"))
 
 
 class Router(nn.Module):
@@ -141,11 +149,6 @@ class Router(nn.Module):
             raise ValueError("num_choices_per_token must be in [1, num_choices].")
         if gate_mode not in ("renorm", "switch"):
             raise ValueError(f"gate_mode must be 'renorm' or 'switch', got {gate_mode!r}.")
-        if noise_mlp_hidden_dims is not None:
-            raise NotImplementedError(
-                "router exploration noise (noise_mlp_hidden_dims) is training-loop state "
-                "that this implementation does not build; construct the router without it"
-            )
         self.feature_dim = feature_dim
         self.num_choices = num_choices
         self.num_choices_per_token = num_choices_per_token
@@ -154,17 +157,50 @@ class Router(nn.Module):
         self.gate_mode = gate_mode
         self.score_mlp = ScoreMLP(feature_dim, score_mlp_hidden_dims, num_choices,
                                   score_mlp_activation)
-        self.noise_mlp = None
+        # ``None`` (this build's default) leaves the router without a noise head:
+        # deterministic in training mode too.  The reference always builds one.
+        self.noise_mlp = (
+            ScoreMLP(feature_dim, noise_mlp_hidden_dims, num_choices, noise_mlp_activation)
+            if noise_mlp_hidden_dims is not None else None
+        )
         self.register_buffer("choice_bias", torch.zeros(num_choices))
+        # NESTOR_ROUTER_NOISE_ANNEAL_STEPS=N: the noise decays linearly to zero over the
+        # first N training forwards (nestor/backbones/nestor.py:469-484); the counter is
+        # a persistent buffer so that it survives a resume.
+        self._noise_anneal_steps = _anneal_steps_from_env()
+        if self._noise_anneal_steps > 0:
+            self.register_buffer("_noise_steps", torch.zeros((), dtype=torch.long))
+
+    def draw_noise(self, batch_size: int, seq_len: int, device, dtype: torch.dtype) -> Tensor:
+        """The standard-normal factor of the exploration noise, ``[B, S, C]``: drawn
+        outside an activation checkpoint and passed to ``forward(noise=...)`` it makes
+        the recompute route exactly as the forward did
+        (nestor/backbones/nestor.py:486-518)."""
+
+        return torch.randn(batch_size, seq_len, self.num_choices, device=device, dtype=dtype)
+
+    def _explore(self, x: Tensor, scores: Tensor, noise: Tensor | None) -> Tensor:
+        if not (self.training and self.noise_mlp is not None):
+            return scores
+        eps = torch.randn_like(scores) if noise is None else noise.to(scores.dtype)
+        perturbation = eps * F.softplus(self.noise_mlp(x))
+        if self._noise_anneal_steps > 0:
+            done = (self._noise_steps.float() / self._noise_anneal_steps).clamp(max=1.0)
+            perturbation = perturbation * (1.0 - done)
+            if not _is_recomputing():
+                self._noise_steps += 1
+        return scores + perturbation
 
     def forward(self, x: Tensor, valid_token_mask: Tensor, noise: Tensor | None = None,
                 scores: Tensor | None = None) -> RouterOutput:
-        """``scores``: the score head's output when the caller already computed it
-        (one GEMM for several heads that read the same rows)."""
+        """``noise``: pre-drawn ``N(0, 1)`` factor of the training noise (``None``: drawn
+        here); ignored outside training mode or without a noise head.  ``scores``: the
+        score head's output when the caller already computed it (one GEMM for several
+        heads that read the same rows)."""
 
-        _refuse_noise(noise)
         if scores is None:
             scores = self.score_mlp(x)
+        scores = self._explore(x, scores, noise)
         probs, topk, gates = route_scores(
             scores, self.choice_bias, self.num_choices_per_token, self.gate_mode, valid_token_mask
         )
@@ -194,9 +230,15 @@ def check_batchable(routers: list[Router]) -> None:
     if not routers:
         raise ValueError("Need at least one router to batch.")
 
+    def mlp_signature(mlp) -> tuple:
+        if mlp is None:
+            return ()
+        return (tuple((l.in_features, l.out_features, l.bias is not None) for l in mlp.layers),
+                mlp.activation)
+
     def signature(r: Router) -> tuple:
-        shape = tuple((l.in_features, l.out_features, l.bias is not None) for l in r.score_mlp.layers)
-        return (r.num_choices, r.num_choices_per_token, r.gate_mode, shape, r.score_mlp.activation)
+        return (r.num_choices, r.num_choices_per_token, r.gate_mode, mlp_signature(r.score_mlp),
+                mlp_signature(r.noise_mlp))
 
     if any(signature(r) != signature(routers[0]) for r in routers[1:]):
         raise ValueError("Private routers differ in shape/gate mode; cannot batch them.")
@@ -232,15 +274,34 @@ def route_private_batched(
     of the stacked tensors, masked to ``valid & member``), stacked gates
     ``[B, S, G, Q]`` and stacked choices ``[B, S, G, k]``.  ``scores``
     (``[B*S, G*Q]``, head-major) skips the score GEMM when the caller has it.
-    ``training`` changes nothing here (it only gates the noise, which is refused)."""
+    ``training`` with noise heads: every router's scores are perturbed as in
+    ``Router.forward``, from ONE draw ``[B, S, G, Q]`` (or the pre-drawn ``noise``) and
+    one batched noise-head GEMM; each router's anneal counter advances as it would
+    alone (nestor/backbones/batched_router.py:188-208)."""
 
-    _refuse_noise(noise)
     first = routers[0]
     groups = len(routers)
     batch, seq, dim = x.shape
+    flat_x = x.reshape(batch * seq, dim)
     if scores is None:
-        scores = batched_mlp(x.reshape(batch * seq, dim), [r.score_mlp for r in routers])
+        scores = batched_mlp(flat_x, [r.score_mlp for r in routers])
     scores = scores.reshape(batch, seq, groups, first.num_choices)
+    if training and first.noise_mlp is not None:
+        spread = F.softplus(batched_mlp(flat_x, [r.noise_mlp for r in routers]).view_as(scores))
+        eps = torch.randn_like(scores) if noise is None else noise.to(scores.dtype)
+        perturbation = eps * spread
+        if any(r._noise_anneal_steps > 0 for r in routers):
+            done = torch.stack([
+                (r._noise_steps.float() / r._noise_anneal_steps).clamp(max=1.0)
+                if r._noise_anneal_steps > 0 else torch.zeros((), device=x.device)
+                for r in routers
+            ])
+            perturbation = perturbation * (1.0 - done).to(perturbation.dtype)[None, None, :, None]
+            if not _is_recomputing():
+                for r in routers:
+                    if r._noise_anneal_steps > 0:
+                        r._noise_steps += 1
+        scores = scores + perturbation
     bias = torch.stack([r.choice_bias for r in routers])
     member = valid_token_mask.unsqueeze(-1) & group_active_mask
     probs, topk, gates = route_scores(

@@ -1,4 +1,5 @@
-"""Router and slot-construction oracles (eval mode, single-linear score heads)."""
+"""Router and slot-construction oracles (single-linear score heads; the training-mode
+exploration noise as a function of a given standard-normal draw)."""
 
 from __future__ import annotations
 
@@ -24,6 +25,19 @@ def stable_topk(values: Tensor, k: int) -> Tensor:
     (whose tie order is unspecified) that both sides of every parity test share."""
 
     return torch.sort(values, dim=-1, descending=True, stable=True).indices[..., :k]
+
+
+def explore(scores: Tensor, eps: Tensor, noise_head: Tensor, steps_done: float = 0.0,
+            anneal_steps: int = 0) -> Tensor:
+    """Training-mode scores of a router with a noise head
+    (nestor/backbones/nestor.py:540-556; batched: batched_router.py:188-208):
+    ``scores + eps * softplus(noise_head) * (1 - min(steps_done / anneal_steps, 1))``,
+    with ``eps`` the standard-normal draw, ``noise_head = noise_mlp(x)`` and the anneal
+    factor 1 when ``anneal_steps`` is 0.  Written with log1p/exp, not ``F.softplus``."""
+
+    spread = torch.where(noise_head > 20, noise_head, torch.log1p(torch.exp(noise_head.clamp(max=20))))
+    keep = 1.0 if anneal_steps <= 0 else 1.0 - min(steps_done / anneal_steps, 1.0)
+    return scores + eps * spread * keep
 
 
 def route(

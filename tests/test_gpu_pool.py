@@ -203,3 +203,49 @@ def test_pool_compiles_as_one_graph(cuda, layout):
         assert (gp0[n] is None) == (gp1[n] is None), n
         if gp0[n] is not None:
             assert torch.equal(gp0[n], gp1[n]), n
+
+
+def test_pool_with_router_noise_under_checkpoint_recompute(cuda):
+    """Exploration noise pre-drawn with ``draw_router_noise`` and passed as ``router_noise``
+    (nestor/backbones/expert_pools.py:588-623): the checkpoint's recompute routes as the
+    forward did, so outputs and gradients equal the run without a checkpoint bit for bit;
+    without noise heads the same call is the deterministic pool."""
+
+    import nestor_amd as na
+    from torch.utils.checkpoint import checkpoint
+
+    x, valid, gates, active, _ = _inputs(cuda)
+    torch.manual_seed(5)
+    pool = na.ExpertPoolMLP(40, 4, 2, 3, 1, 5, 1, [], router_noise_mlp_hidden_dims=[],
+                            private_gate_mode="switch")
+    with torch.no_grad():
+        pool.path_gate.weight.normal_()
+        for r in [pool.public_router, *pool.private_routers]:
+            r.noise_mlp.layers[0].weight.normal_(std=0.5)
+    assert na.consolidate_stacked_expert_banks(pool, force=True) == 2
+    pool.triton_fused = pool.triton_index = pool.fused_gate = True
+    pool = pool.to(cuda).train()
+    noise = pool.draw_router_noise(3, 70, cuda, torch.bfloat16)
+
+    def run(use_checkpoint, router_noise):
+        for p in pool.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            fn = lambda a: pool(a, valid, gates, active, router_noise=router_noise)[0]
+            out = checkpoint(fn, xi, use_reentrant=False) if use_checkpoint else fn(xi)
+        out.float().square().sum().backward()
+        return out.detach(), xi.grad, {n: p.grad.clone() for n, p in pool.named_parameters() if p.grad is not None}
+
+    out0, gx0, gp0 = run(False, noise)
+    out1, gx1, gp1 = run(True, noise)
+    assert torch.equal(out0, out1) and torch.equal(gx0, gx1)
+    assert gp0.keys() == gp1.keys() and all(torch.equal(gp0[n], gp1[n]) for n in gp0)
+    assert any("noise_mlp" in n for n in gp0)          # the noise heads learn
+    # another draw routes differently; evaluation mode ignores the draw
+    other = {k: -v for k, v in noise.items()}
+    assert not torch.equal(run(False, other)[0], out0)
+    pool.eval()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        assert torch.equal(pool(x, valid, gates, active, router_noise=noise)[0],
+                           pool(x, valid, gates, active)[0])

@@ -207,3 +207,101 @@ def test_balancing_counts_and_bias_update(cuda, n, choices, k):
     before = router.choice_bias.cpu().clone()
     router.update_detached_parameters(topk.to(cuda), valid.to(cuda))
     assert torch.equal(router.choice_bias.cpu(), orouter.balancing_update(before, topk, valid, 0.01))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mode,k", [("renorm", 2), ("switch", 1)])
+def test_router_exploration_noise(cuda, dtype, mode, k):
+    """Training-mode routers with a noise head (nestor/backbones/nestor.py:540-556): the
+    scores are ``score + eps * softplus(noise head)`` for the draw handed in, the
+    selection is the oracle's on those scores, evaluation mode and a router without a
+    noise head ignore the draw, the noise head receives a gradient, and an own draw
+    follows the RNG seed."""
+
+    import nestor_amd as na
+
+    torch.manual_seed(0)
+    router = na.Router(48, 8, k, [], noise_mlp_hidden_dims=[], gate_mode=mode).to(cuda).to(dtype)
+    with torch.no_grad():
+        router.choice_bias.normal_(std=0.1)
+        router.noise_mlp.layers[0].weight.normal_(std=0.3)
+    g = torch.Generator(device=cuda).manual_seed(4)
+    x = torch.randn(3, 50, 48, generator=g, device=cuda, dtype=dtype)
+    valid = torch.rand(3, 50, generator=g, device=cuda) > 0.1
+    eps = router.draw_noise(3, 50, cuda, dtype)
+    router.train()
+    out = router(x, valid, noise=eps)
+    plain = router.score_mlp(x)
+    head = router.noise_mlp(x)
+    want_scores = orouter.explore(plain.cpu().double(), eps.cpu().double(), head.cpu().double())
+    if dtype == torch.bfloat16:   # softplus, product and sum each round to 8 bits
+        torch.testing.assert_close(out.scores.cpu().double(), want_scores, rtol=2 ** -6, atol=4e-2)
+    else:
+        torch.testing.assert_close(out.scores.cpu().double(), want_scores, rtol=1e-5, atol=1e-5)
+    assert not torch.equal(out.scores, plain)
+    want = orouter.route(out.scores.cpu(), router.choice_bias.cpu(), k, mode, valid.cpu(),
+                         softmax_dtype=torch.float32)
+    assert torch.equal(out.topk_indices.cpu(), want.topk_indices)
+    assert torch.equal(out.active_mask.cpu(), want.active_mask) or dtype == torch.bfloat16
+    # the noise head learns: its weight gets a gradient through the perturbed scores
+    (out.softmax_probs.float() * torch.arange(8, device=cuda)).sum().backward()
+    assert router.noise_mlp.layers[0].weight.grad.abs().sum() > 0
+    # an own draw follows the seed
+    torch.manual_seed(7)
+    a = router(x, valid).scores
+    torch.manual_seed(7)
+    b = router(x, valid).scores
+    assert torch.equal(a, b) and not torch.equal(a, out.scores)
+    # evaluation mode, and a router without a noise head, are deterministic
+    router.eval()
+    assert torch.equal(router(x, valid, noise=eps).scores, plain)
+    bare = na.Router(48, 8, k, [], gate_mode=mode).to(cuda).to(dtype).train()
+    assert torch.equal(bare(x, valid, noise=eps).scores, bare.score_mlp(x))
+
+
+def test_batched_noisy_routers_equal_one_router_at_a_time(cuda, monkeypatch):
+    """``route_private_batched`` in training mode: one draw ``[B, S, G, Q]`` gives every
+    router the result it gets alone on its slab, and with the anneal schedule on each
+    counter advances once per forward but not inside a backward recompute
+    (nestor/backbones/batched_router.py:188-208, nestor.py:548-555)."""
+
+    import nestor_amd as na
+
+    monkeypatch.setenv("NESTOR_ROUTER_NOISE_ANNEAL_STEPS", "4")
+    torch.manual_seed(1)
+    routers = [na.Router(32, 4, 1, [], noise_mlp_hidden_dims=[], gate_mode="switch").to(cuda)
+               for _ in range(3)]
+    for r in routers:
+        with torch.no_grad():
+            r.noise_mlp.layers[0].weight.normal_(std=0.5)
+        r.train()
+        assert int(r._noise_steps) == 0
+    g = torch.Generator(device=cuda).manual_seed(2)
+    x = torch.randn(2, 40, 32, generator=g, device=cuda)
+    valid = torch.ones(2, 40, dtype=torch.bool, device=cuda)
+    member = torch.rand(2, 40, 3, generator=g, device=cuda) > 0.3
+    eps = torch.randn(2, 40, 3, 4, generator=g, device=cuda)
+    outs, gates, topk = na.route_private_batched(routers, x, valid, member, training=True, noise=eps)
+    assert [int(r._noise_steps) for r in routers] == [1, 1, 1]
+    for r in routers:
+        r._noise_steps.zero_()
+    for gi, r in enumerate(routers):
+        alone = r(x, valid & member[:, :, gi], noise=eps[:, :, gi])
+        torch.testing.assert_close(outs[gi].scores, alone.scores, rtol=1e-5, atol=1e-6)
+        assert torch.equal(outs[gi].topk_indices, alone.topk_indices)
+    # step 1 of 4: three quarters of the perturbation; step 4 and later: none
+    full = orouter.explore(routers[0].score_mlp(x).detach().cpu().double(), eps[:, :, 0].cpu().double(),
+                           routers[0].noise_mlp(x).detach().cpu().double())
+    base = routers[0].score_mlp(x).detach().cpu().double()
+    step1 = routers[0](x, valid, noise=eps[:, :, 0]).scores.detach().cpu().double()
+    torch.testing.assert_close(step1 - base, 0.75 * (full - base), rtol=1e-4, atol=1e-5)
+    routers[0]._noise_steps.fill_(9)
+    assert torch.equal(routers[0](x, valid, noise=eps[:, :, 0]).scores, routers[0].score_mlp(x))
+    # a checkpoint's recompute does not advance the schedule
+    from torch.utils.checkpoint import checkpoint
+
+    routers[1]._noise_steps.zero_()
+    xi = x.clone().requires_grad_(True)
+    out = checkpoint(lambda a: routers[1](a, valid, noise=eps[:, :, 1]).softmax_probs, xi, use_reentrant=False)
+    out.sum().backward()
+    assert int(routers[1]._noise_steps) == 1

@@ -165,28 +165,45 @@ def test_flop_counter_sees_the_expert_gemms():
         assert counter.get_total_flops() == 2 * tokens * d * 32
 
 
-def test_training_noise_is_refused_not_ignored():
-    """Exploration noise belongs to the training loop and is not built; asking for it
-    raises instead of silently routing without it."""
+def test_router_noise_heads_are_built_and_batchable():
+    """Routers take the reference's noise head (nestor/backbones/nestor.py:459-466); a pool
+    hands ``router_noise_mlp_hidden_dims`` to every router, and batching needs same-shaped
+    noise heads as it needs same-shaped score heads (batched_router.py:71-94)."""
 
-    with pytest.raises(NotImplementedError):
-        na.Router(16, 4, 1, [], noise_mlp_hidden_dims=[8])
-    with pytest.raises(NotImplementedError):
-        na.ExpertPoolMLP(16, 2, 1, 2, 1, 2, 1, [], router_noise_mlp_hidden_dims=[8])
-    router = na.Router(16, 4, 1, [])
-    with pytest.raises(NotImplementedError):
-        router(torch.zeros(1, 2, 16), torch.ones(1, 2, dtype=torch.bool), noise=torch.zeros(1, 2, 4))
-    pool = na.ExpertPoolMLP(16, 2, 1, 2, 1, 2, 1, [])
-    args = (torch.zeros(1, 2, 16), torch.ones(1, 2, dtype=torch.bool), torch.zeros(1, 2, 2),
-            torch.ones(1, 2, 2, dtype=torch.bool))
-    for call in (pool.forward, pool.forward_per_group):
-        with pytest.raises(NotImplementedError):
-            call(*args, router_noise=torch.zeros(1))
-    with pytest.raises(NotImplementedError):
-        pool.forward_per_slot(*args, torch.zeros(1, 2, 1, dtype=torch.long), router_noise=torch.zeros(1))
-    with pytest.raises(NotImplementedError):
-        na.route_private_batched(list(pool.private_routers), args[0], args[1], args[3], training=True,
-                                 noise=torch.zeros(1))
+    router = na.Router(16, 4, 1, [], noise_mlp_hidden_dims=[8])
+    assert [tuple(l.weight.shape) for l in router.noise_mlp.layers] == [(8, 16), (4, 8)]
+    assert na.Router(16, 4, 1, []).noise_mlp is None
+    assert tuple(router.draw_noise(2, 3, "cpu", torch.float32).shape) == (2, 3, 4)
+    pool = na.ExpertPoolMLP(16, 2, 1, 2, 1, 2, 1, [], router_noise_mlp_hidden_dims=[])
+    assert pool.public_router.noise_mlp is not None
+    assert all(r.noise_mlp is not None for r in pool.private_routers)
+    drawn = pool.draw_router_noise(2, 3, "cpu", torch.float32)
+    assert tuple(drawn["private"].shape) == (2, 3, 2, 2) and tuple(drawn["public"].shape) == (2, 3, 2)
+    from nestor_amd.router import check_batchable
+
+    with pytest.raises(ValueError):
+        check_batchable([na.Router(16, 4, 1, [], noise_mlp_hidden_dims=[8]), na.Router(16, 4, 1, [])])
+    # the anneal counter is a buffer only when the schedule is on
+    assert not hasattr(router, "_noise_steps")
+
+
+def test_oracle_exploration_formula():
+    """``oracle.router.explore`` against the textbook pieces: softplus by its definition in
+    fp64, the anneal factor at its corners, and linearity in the draw."""
+
+    from oracle import router as orouter
+
+    g = torch.Generator().manual_seed(3)
+    scores, eps, head = (torch.randn(5, 7, generator=g, dtype=torch.float64) for _ in range(3))
+    head[0, 0], head[0, 1] = 40.0, -40.0
+    want = scores + eps * torch.log(1 + torch.exp(head))
+    assert torch.allclose(orouter.explore(scores, eps, head), want, rtol=1e-12, atol=1e-12)
+    assert torch.equal(orouter.explore(scores, torch.zeros_like(eps), head), scores)
+    assert torch.equal(orouter.explore(scores, eps, head, 10, 10), scores)          # fully annealed
+    assert torch.equal(orouter.explore(scores, eps, head, 25, 10), scores)          # clamped
+    half = orouter.explore(scores, eps, head, 5, 10)
+    assert torch.allclose(half - scores, 0.5 * (want - scores), rtol=1e-12, atol=1e-12)
+    assert torch.allclose(orouter.explore(scores, 2 * eps, head) - scores, 2 * (want - scores))
 
 
 def test_bf16_shadow_follows_data_writes():
